@@ -1,0 +1,76 @@
+// Shared device/host helpers for the gfx950 (MI355X, CDNA4) kernels of this library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace msd {
+
+// ---- vector types -------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+// ---- error codes returned by every extern "C" entry point ----------------------------
+enum : int {
+  MSD_OK = 0,
+  MSD_ERR_BAD_ARG = 1,      // null pointer, non-positive size, unsupported head_dim/dtype
+  MSD_ERR_UNSUPPORTED = 2,  // shape or option outside what the kernels implement
+  MSD_ERR_WORKSPACE = 3,    // workspace too small
+  MSD_ERR_LAUNCH = 4,       // hipLaunch / runtime error (hipGetLastError != hipSuccess)
+};
+
+enum : int { MSD_DTYPE_BF16 = 0, MSD_DTYPE_F16 = 1 };
+
+// ---- element traits: 16-bit storage type -> MFMA operand type + builtins -------------
+template <int DT>
+struct Elem;
+template <>
+struct Elem<MSD_DTYPE_BF16> {
+  typedef __bf16 type;
+  typedef bf16x8_t x8;
+  typedef bf16x4_t x4;
+  static __device__ __forceinline__ f32x16_t mfma32(x8 a, x8 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ type from_float(float f) { return (__bf16)f; }
+};
+template <>
+struct Elem<MSD_DTYPE_F16> {
+  typedef _Float16 type;
+  typedef f16x8_t x8;
+  typedef f16x4_t x4;
+  static __device__ __forceinline__ f32x16_t mfma32(x8 a, x8 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ type from_float(float f) { return (_Float16)f; }
+};
+
+// LDS pointer in address space 3 (needed by the transposing LDS read builtin).
+#define MSD_LDS __attribute__((address_space(3)))
+
+// One ds_read_b64_tr_b16: the 16 lanes of a quarter-wave each point at 4 consecutive
+// 16-bit elements; viewing those 64 elements as a 4 x 16 matrix (row j = lanes 4j..4j+3),
+// lane i receives column i (4 elements, one from each row).
+__device__ __forceinline__ s16x4_t lds_read_tr16(const void* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)(uintptr_t)(p));
+}
+
+// Exchange a value with the lane 32 positions away (the other half of the wavefront).
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// round-to-nearest-even fp32 -> bf16 bits, then back to fp32 (used where a rounding point
+// of the reference arithmetic has to be reproduced exactly)
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
+
+}  // namespace msd
