@@ -64,8 +64,31 @@ __device__ __forceinline__ s16x4_t lds_read_tr16(const void* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)(uintptr_t)(p));
 }
 
-// Exchange a value with the lane 32 positions away (the other half of the wavefront).
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Combine a value with the one held by the lane 32 positions away (the other half of the
+// wavefront) using v_permlane32_swap: after the swap one result register holds lanes 0..31 of
+// the input in both halves and the other holds lanes 32..63 in both halves.
+// (Written as inline asm: with the builtin the optimiser of this toolchain folds the second
+// result into the first when both inputs hold the same value.  The leading s_nop covers the
+// VALU-write -> permlane-swap hazard that the compiler cannot see inside an asm block.)
+__device__ __forceinline__ void half_swap(float v, float& lo, float& hi) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  lo = a;
+  hi = b;
+}
+__device__ __forceinline__ float half_max(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_sum(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return lo + hi;
+}
+
+// Lazy-rescale threshold of the online softmax, in log2 units.
+constexpr float kTau = 8.0f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -61,14 +61,30 @@ struct FaCfg {
   static constexpr int kOutStageBytes = NWAVES * 32 * kORowBytes;
   // K/V double buffered; the output staging reuses the same memory after the last tile
   static constexpr int kLdsBytes = 2 * kStageBytes > kOutStageBytes ? 2 * kStageBytes : kOutStageBytes;
-  static constexpr int kChunksPerThread = BN * 16 / kNT;  // 16-byte chunks of one tile per thread
-  static_assert(BN * 16 % kNT == 0, "tile must split evenly over the threads");
+  static constexpr int kGroupsPerWave = BN / 4 / NWAVES;  // 4-row (1 KiB) LDS-DMA groups per wave and tile
+  static_assert(BN % (4 * NWAVES) == 0, "tile must split evenly over the wavefronts");
 };
+
+#if defined(__HIP_DEVICE_COMPILE__)
+// LDS-DMA of one K tile and one V tile: every wave issues G pairs of 1 KiB transfers.
+template <int G, int NWAVES>
+__device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu_buffer_rsrc_t v_rsrc,
+                                         MSD_LDS char* kb, MSD_LDS char* vb, const int (&k_voff)[G],
+                                         const int (&v_voff)[G], int wave, int k_soff, int v_soff) {
+#pragma unroll
+  for (int i = 0; i < G; ++i) {
+    const int g = i * NWAVES + wave;  // 4-row group of the tile
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g * 1024), 16, k_voff[i], k_soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g * 1024), 16, v_voff[i], v_soff, 0, 0);
+  }
+}
+#endif
 
 // Register budget: 8 wavefronts per CU (two per SIMD) in every configuration, i.e. at most 256
 // registers per lane; the 4-wave configurations run two workgroups per CU.
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
   using E = Elem<DT>;
   using T = typename E::type;
@@ -78,7 +94,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int h = lane >> 5;
 
@@ -139,38 +155,35 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int r = 0; r < 16; ++r) oacc[db][qb][r] = 0.f;
   }
 
-  // ---- global -> register -> LDS staging of one K/V tile ----------------------------------------
-  i32x4_t kreg[C::kChunksPerThread], vreg[C::kChunksPerThread];
+  // ---- global -> LDS staging of one K/V tile (LDS-DMA, no registers) ------------------------------
+  // One buffer_load_dwordx4 ... lds moves 64 x 16 bytes: lane L's 16 bytes land at lds_base + 16*L,
+  // i.e. one instruction fills 4 consecutive 256-byte rows.  The swizzles are applied on the
+  // global side: the lane that fills physical chunk pc of a row fetches the logical chunk
+  // pc ^ swizzle(row).  The per-lane byte offset inside a tile never changes; the tile position
+  // is a scalar offset.  Rows past the end of the sequence are out of the buffer's range and read
+  // as zeros (their scores are masked to -inf below).
   auto tile_key0 = [&](int t) -> int {
     if (SPARSE) return sel[t / kSub] * 128 + (t % kSub) * BN;
     return t * BN;
   };
-  auto load_tile = [&](int t) {
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)kg, 0, (int)(((long long)(p.Skv - 1) * p.k_ss + C::kD) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)vg, 0, (int)(((long long)(p.Skv - 1) * p.v_ss + C::kD) * 2), 0x00020000);
+  const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
+  int k_voff[C::kGroupsPerWave], v_voff[C::kGroupsPerWave];
+#pragma unroll
+  for (int i = 0; i < C::kGroupsPerWave; ++i) {
+    const int row = 4 * (i * NWAVES + wave) + (lane >> 4);
+    const int pc = lane & 15;
+    k_voff[i] = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
+    v_voff[i] = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
+  }
+  auto load_tile = [&](int t, int stage) {
     const int key0 = tile_key0(t);
-#pragma unroll
-    for (int i = 0; i < C::kChunksPerThread; ++i) {
-      const int c = i * C::kNT + tid;
-      const int row = c >> 4, c16 = c & 15;
-      const int key = key0 + row;
-      const bool ok = key < p.Skv;
-      const long long kr = (long long)(ok ? key : 0);
-      i32x4_t kk = *(const i32x4_t*)(kg + kr * p.k_ss + c16 * 8);
-      i32x4_t vv = *(const i32x4_t*)(vg + kr * p.v_ss + c16 * 8);
-      if (!ok) { kk = i32x4_t{0, 0, 0, 0}; vv = i32x4_t{0, 0, 0, 0}; }
-      kreg[i] = kk;
-      vreg[i] = vv;
-    }
-  };
-  auto store_tile = [&](int stage) {
     MSD_LDS char* kb = smem + stage * C::kStageBytes;
-    MSD_LDS char* vb = kb + C::kTileBytes;
-#pragma unroll
-    for (int i = 0; i < C::kChunksPerThread; ++i) {
-      const int c = i * C::kNT + tid;
-      const int row = c >> 4, c16 = c & 15;
-      *(MSD_LDS i32x4_t*)(kb + row * C::kRowBytes + ((c16 ^ (row & 15)) << 4)) = kreg[i];
-      *(MSD_LDS i32x4_t*)(vb + row * C::kRowBytes + ((c16 ^ ((row & 3) << 2)) << 4)) = vreg[i];
-    }
+    tile_dma<C::kGroupsPerWave, NWAVES>(k_rsrc, v_rsrc, kb, kb + C::kTileBytes, k_voff, v_voff, wave,
+                                        key0 * k_row_bytes, key0 * v_row_bytes);
   };
 
   // per-lane constant parts of the LDS read addresses
@@ -183,20 +196,18 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int v_row_off = v_key * C::kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
   const int v_swz = (lane & 15) >> 2;
 
-  if (n_tiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
+  if (n_tiles > 0) load_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
 
   for (int t = 0; t < n_tiles; ++t) {
     const int stage = t & 1;
-    if (t + 1 < n_tiles) load_tile(t + 1);
+    if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
 
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
     MSD_LDS const char* vb_base = kb_base + C::kTileBytes;
 
-    // ---- S^T = K Q^T -------------------------------------------------------------------------
+    // ---- S^T = K Q^T: kNKB independent accumulation chains per 16-wide step of head_dim -------
     f32x16_t sacc[C::kNKB][C::kNQB];
 #pragma unroll
     for (int kb = 0; kb < C::kNKB; ++kb)
@@ -204,15 +215,34 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int qb = 0; qb < C::kNQB; ++qb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[kb][qb][r] = 0.f;
+    X8 afrag[2][C::kNKB];
 #pragma unroll
-    for (int kb = 0; kb < C::kNKB; ++kb) {
+    for (int kb = 0; kb < C::kNKB; ++kb)
+      afrag[0][kb] = *(MSD_LDS const X8*)(kb_base + kb * 32 * C::kRowBytes + k_row_off + ((h ^ k_swz) << 4));
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const X8 a = *(MSD_LDS const X8*)(kb_base + kb * 32 * C::kRowBytes + k_row_off +
-                                          (((2 * ks + h) ^ k_swz) << 4));
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks + 1 < 8) {
 #pragma unroll
-        for (int qb = 0; qb < C::kNQB; ++qb) sacc[kb][qb] = E::mfma32(a, qf[qb][ks], sacc[kb][qb]);
+        for (int kb = 0; kb < C::kNKB; ++kb)
+          afrag[(ks + 1) & 1][kb] = *(MSD_LDS const X8*)(kb_base + kb * 32 * C::kRowBytes + k_row_off +
+                                                         (((2 * (ks + 1) + h) ^ k_swz) << 4));
       }
+#pragma unroll
+      for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+        for (int qb = 0; qb < C::kNQB; ++qb)
+          sacc[kb][qb] = E::mfma32(afrag[ks & 1][kb], qf[qb][ks], sacc[kb][qb]);
+    }
+    if (SCHED == 1) {
+      // operand reads run one head_dim step ahead of the matrix instructions that consume them
+      __builtin_amdgcn_sched_group_barrier(0x100, C::kNKB, 0);
+#pragma unroll
+      for (int ks = 0; ks < 7; ++ks) {
+        __builtin_amdgcn_sched_group_barrier(0x100, C::kNKB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, C::kNKB * C::kNQB, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, C::kNKB * C::kNQB, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- mask keys past the end of the sequence (last tile only) --------------------------------
@@ -230,7 +260,10 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         }
     }
 
-    // ---- online softmax; P^T is packed in place as the B operand of the second product ----------
+    // ---- online softmax in the exp2 domain with a lazily updated reference maximum --------------
+    // m_run is the reference (scaled by scale*log2 e) that the running sum and the accumulator are
+    // expressed in.  It only moves when some row's new maximum exceeds it by more than kTau, so
+    // the accumulator rescale is skipped for almost every tile; probabilities stay <= 2^kTau.
     X8 pf[C::kNQB][C::kNKB][2];
 #pragma unroll
     for (int qb = 0; qb < C::kNQB; ++qb) {
@@ -239,11 +272,18 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][qb][r]);
-      mx = fmaxf(mx, xor32(mx));
-      const float m_new = fmaxf(m_run[qb], mx);
-      const float mc = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
-      const float alpha = fast_exp2(m_run[qb] * p.scale_log2 - mc);
-      m_run[qb] = m_new;
+      mx = half_max(mx) * p.scale_log2;
+      if (__builtin_amdgcn_ballot_w64(mx > m_run[qb] + kTau) != 0) {
+        const float m_new = fmaxf(m_run[qb], mx);
+        const float alpha = fast_exp2(m_run[qb] - (m_new == -INFINITY ? 0.f : m_new));
+        m_run[qb] = m_new;
+        l_run[qb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[db][qb][r] *= alpha;
+      }
+      const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
       float ls = 0.f;
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb) {
@@ -261,11 +301,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
           pf[qb][kb][t2] = pk;
         }
       }
-      l_run[qb] = l_run[qb] * alpha + ls;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][qb][r] *= alpha;
+      l_run[qb] += ls;
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------------------
@@ -289,7 +325,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       }
     }
 
-    if (t + 1 < n_tiles) store_tile(stage ^ 1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): next tile's LDS-DMA issued by this wave is complete
     __syncthreads();
   }
 
@@ -300,12 +336,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
 #pragma unroll
   for (int qb = 0; qb < C::kNQB; ++qb) {
-    const float l_tot = l_run[qb] + xor32(l_run[qb]);
+    const float l_tot = half_sum(l_run[qb]);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int qrow_l = q0 + wave * QPW + qb * 32 + l32;
     if (p.lse && h == 0 && qrow_l < p.Sq) {
       const long long li = ((long long)b * p.N + n) * p.Sq + qrow_l;
-      p.lse[li] = l_tot > 0.f ? m_run[qb] * p.scale + __logf(l_tot) : -INFINITY;
+      p.lse[li] = l_tot > 0.f ? m_run[qb] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
     }
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -333,12 +369,13 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
     __builtin_amdgcn_wave_barrier();
   }
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
-  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE>;
+  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED>;
   static bool configured = false;  // raising the dynamic LDS limit is idempotent
   if (!configured) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) !=
@@ -359,9 +396,10 @@ using namespace msd;
 
 extern "C" {
 
-// Tuning hook used by the benchmark sweep: selects the dense kernel variant
-// (0: 8 waves x 32 rows, 128-key tiles; 1: 4 waves x 32 rows, 64-key tiles;
-//  2: 4 waves x 64 rows, 64-key tiles; 3: 8 waves x 32 rows, 64-key tiles).
+// Tuning hook used by benchmark sweeps: selects the dense kernel variant
+// (0, default: 8 waves x 32 rows, 128-key tiles, operand reads scheduled one step ahead;
+//  1: 4 waves x 32 rows, 64-key tiles, compiler scheduling; 2: as 0 with compiler scheduling;
+//  3: as 1 with scheduled operand reads).
 static int g_dense_variant = 0;
 void mindiesd_set_dense_variant(int v) { g_dense_variant = v; }
 
@@ -373,6 +411,9 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   if (!q || !k || !v || !out) return MSD_ERR_BAD_ARG;
   if (B <= 0 || N <= 0 || Nkv <= 0 || Sq <= 0 || Skv <= 0 || N % Nkv != 0) return MSD_ERR_BAD_ARG;
   if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (!(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
+  // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
+  if ((long long)Skv * k_ss * 2 >= (1ll << 31) || (long long)Skv * v_ss * 2 >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
   // 16-byte vector accesses: every row start must be 16-byte aligned
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
@@ -388,13 +429,13 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   p.scale_log2 = scale * 1.4426950408889634f;
   if (dtype == MSD_DTYPE_BF16) {
     switch (g_dense_variant) {
-      case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false>(p, stream);
-      case 2: return launch_fa<MSD_DTYPE_BF16, 4, 64, 64, false>(p, stream);
-      case 3: return launch_fa<MSD_DTYPE_BF16, 8, 32, 64, false>(p, stream);
-      default: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false>(p, stream);
+      case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);
+      case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
+      case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);
+      default: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1>(p, stream);
     }
   }
-  return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1>(p, stream);
 }
 
 }  // extern "C"

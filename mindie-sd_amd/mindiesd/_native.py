@@ -1,0 +1,61 @@
+"""ctypes binding of ``plugin/libmindiesd_hip.so`` (C ABI declared in include/mindiesd_hip.h).
+
+The library location mirrors the reference's ``<package>/plugin/libPTAExtensionOPS.so``
+(mindiesd/layers/register_ops.py:24-44).  Importing the package never loads it; the first
+fused call does, and a missing library is a hard error -- there is no CPU fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "plugin", "libmindiesd_hip.so")
+_lib = None
+
+ERRORS = {
+    1: "bad argument (null/misaligned pointer, non-positive size, unsupported dtype)",
+    2: "unsupported shape or option",
+    3: "workspace too small",
+    4: "HIP launch failure",
+}
+
+c_int, c_ll, c_f, c_p, c_sz = ctypes.c_int, ctypes.c_longlong, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/mindiesd_hip.h
+SIGNATURES = {
+    "mindiesd_flash_attention_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p]),
+    "mindiesd_set_dense_variant": (None, [c_int]),
+}
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+def lib():
+    """Load (once) and return the HIP library; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(_LIB_PATH):
+            raise RuntimeError(
+                f"mindiesd HIP library not found at {_LIB_PATH}; build it with "
+                f"`python mindie-sd_amd/build.py` (there is no CPU fallback for fused ops)")
+        handle = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed: {ERRORS.get(rc, 'error')} (code {rc})")
+
+
+def stream_ptr(device=None):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}
