@@ -104,7 +104,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int per_xcd = (total + 7) / 8;
   int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
-  if (SPARSE && p.order) work = p.order[work];
+  if (SPARSE && p.order) work = p.order[blockIdx.x < total ? blockIdx.x : 0];
+  if (SPARSE && p.order && blockIdx.x >= total) return;
   const int bn = work / q_tiles;
   const int qt = work - bn * q_tiles;
   const int b = bn / p.N;
@@ -403,30 +404,63 @@ extern "C" {
 static int g_dense_variant = 0;
 void mindiesd_set_dense_variant(int v) { g_dense_variant = v; }
 
+static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
+                        int Nkv, int Sq, int Skv, int D, const long long* st, float scale) {
+  if (!q || !k || !v || !out) return MSD_ERR_BAD_ARG;
+  if (B <= 0 || N <= 0 || Nkv <= 0 || Sq <= 0 || Skv <= 0 || N % Nkv != 0) return MSD_ERR_BAD_ARG;
+  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (!(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
+  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  // 16-byte vector accesses: every row start must be 16-byte aligned
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
+  long long any = 0;
+  for (int i = 0; i < 12; ++i) any |= st[i];
+  if (any & 7) return MSD_ERR_BAD_ARG;
+  // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
+  if ((long long)Skv * st[5] * 2 >= (1ll << 31) || (long long)Skv * st[8] * 2 >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
+  return MSD_OK;
+}
+
+static FaParams make_params(const void* q, const void* k, const void* v, void* out, float* lse, int B, int N, int Nkv,
+                            int Sq, int Skv, const long long* st, float scale) {
+  FaParams p{};
+  p.q = q; p.k = k; p.v = v; p.o = out; p.lse = lse;
+  p.q_sb = st[0]; p.q_sn = st[1]; p.q_ss = st[2];
+  p.k_sb = st[3]; p.k_sn = st[4]; p.k_ss = st[5];
+  p.v_sb = st[6]; p.v_sn = st[7]; p.v_ss = st[8];
+  p.o_sb = st[9]; p.o_sn = st[10]; p.o_ss = st[11];
+  p.B = B; p.N = N; p.Nkv = Nkv; p.Sq = Sq; p.Skv = Skv;
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  return p;
+}
+
+int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                        int B, int N, int Nkv, int Sq, int Skv, int D, long long q_sb, long long q_sn,
+                                        long long q_ss, long long k_sb, long long k_sn, long long k_ss,
+                                        long long v_sb, long long v_sn, long long v_ss, long long o_sb,
+                                        long long o_sn, long long o_ss, float scale, const int* blk_idx,
+                                        const int* blk_cnt, int kb_stride, const int* order, hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.order = order;
+  p.QB = (Sq + 127) / 128;
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
+}
+
 int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
                                  int B, int N, int Nkv, int Sq, int Skv, int D, long long q_sb, long long q_sn,
                                  long long q_ss, long long k_sb, long long k_sn, long long k_ss, long long v_sb,
                                  long long v_sn, long long v_ss, long long o_sb, long long o_sn, long long o_ss,
                                  float scale, hipStream_t stream) {
-  if (!q || !k || !v || !out) return MSD_ERR_BAD_ARG;
-  if (B <= 0 || N <= 0 || Nkv <= 0 || Sq <= 0 || Skv <= 0 || N % Nkv != 0) return MSD_ERR_BAD_ARG;
-  if (D != 128) return MSD_ERR_UNSUPPORTED;
-  if (!(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
-  // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
-  if ((long long)Skv * k_ss * 2 >= (1ll << 31) || (long long)Skv * v_ss * 2 >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
-  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
-  // 16-byte vector accesses: every row start must be 16-byte aligned
-  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
-  if ((q_sb | q_sn | q_ss | k_sb | k_sn | k_ss | v_sb | v_sn | v_ss | o_sb | o_sn | o_ss) & 7) return MSD_ERR_BAD_ARG;
-  FaParams p{};
-  p.q = q; p.k = k; p.v = v; p.o = out; p.lse = lse;
-  p.q_sb = q_sb; p.q_sn = q_sn; p.q_ss = q_ss;
-  p.k_sb = k_sb; p.k_sn = k_sn; p.k_ss = k_ss;
-  p.v_sb = v_sb; p.v_sn = v_sn; p.v_ss = v_ss;
-  p.o_sb = o_sb; p.o_sn = o_sn; p.o_ss = o_ss;
-  p.B = B; p.N = N; p.Nkv = Nkv; p.Sq = Sq; p.Skv = Skv;
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  const FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   if (dtype == MSD_DTYPE_BF16) {
     switch (g_dense_variant) {
       case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);

@@ -24,6 +24,7 @@ struct Grid3 {
 
 // Source token (t,h,w)-flattened index of position i of the window-ordered image sequence.
 __device__ __forceinline__ int window_source(int i, Grid3 g) {
+  if (g.t == 0) return i;  // identity (plain pooling of an already ordered sequence)
   const int hw = g.h * g.w;
   const int hr = g.h & 7, wr = g.w & 7;
   if (hr == 0 && wr == 0) {
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void rf_rearrange_pool_kernel(const RearrangeP
   const int cnt = min(128, seg_len - seg_blk * 128);
   const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
   const T* src = (const T*)p.src[which] + b * p.s_sb + n * p.s_sn + c16 * 8;
-  T* dst = (T*)p.dst[which] + b * p.d_sb + n * p.d_sn + c16 * 8;
+  T* dst = p.dst[which] ? (T*)p.dst[which] + b * p.d_sb + n * p.d_sn + c16 * 8 : nullptr;
   double acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.0;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void rf_rearrange_pool_kernel(const RearrangeP
     const int from = p.inverse ? pos_perm : pos_orig;
     const int to = p.inverse ? pos_orig : pos_perm;
     const i32x4_t raw = *(const i32x4_t*)(src + (long long)from * p.s_ss);
-    *(i32x4_t*)(dst + (long long)to * p.d_ss) = raw;
+    if (dst) *(i32x4_t*)(dst + (long long)to * p.d_ss) = raw;
     if (p.pool) {
       union { i32x4_t v; T e[8]; } u;
       u.v = raw;
@@ -339,13 +340,15 @@ int mindiesd_rf_rearrange_pool(const void* q, const void* k, const void* v, void
                                long long s_ss, long long d_sb, long long d_sn, long long d_ss, long long p_st,
                                long long p_sb, long long p_sn, long long p_sblk, int t, int h, int w, int txt_len,
                                int inverse, int n_tensors, hipStream_t stream) {
-  if (!q || !q_out || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
-  if (n_tensors < 1 || n_tensors > 3 || (n_tensors > 1 && (!k || !k_out)) || (n_tensors > 2 && (!v || !v_out)))
-    return MSD_ERR_BAD_ARG;
+  if (!q || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+  if (n_tensors < 1 || n_tensors > 3 || (n_tensors > 1 && !k) || (n_tensors > 2 && !v)) return MSD_ERR_BAD_ARG;
+  if (!pool && !q_out) return MSD_ERR_BAD_ARG;  // nothing to produce
   if (D != 128) return MSD_ERR_UNSUPPORTED;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
-  if (t <= 0 || h < 8 || w < 8 || txt_len < 0 || (long long)t * h * w + txt_len != S) return MSD_ERR_BAD_ARG;
-  if ((h % 8 || w % 8) && t < 1) return MSD_ERR_BAD_ARG;
+  // t == 0 selects the identity order (pooling only); otherwise t*h*w image tokens + txt_len text tokens
+  if (txt_len < 0 || t < 0) return MSD_ERR_BAD_ARG;
+  if (t > 0 && (h < 8 || w < 8 || (long long)t * h * w + txt_len != S)) return MSD_ERR_BAD_ARG;
+  if (t == 0 && txt_len > S) return MSD_ERR_BAD_ARG;
   if ((s_sb | s_sn | s_ss | d_sb | d_sn | d_ss) & 7) return MSD_ERR_BAD_ARG;
   RearrangeParams p{};
   p.src[0] = q; p.src[1] = k; p.src[2] = v;

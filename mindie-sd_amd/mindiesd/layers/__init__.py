@@ -1,3 +1,4 @@
-from .flash_attn import attention_forward
+from . import _custom_ops  # noqa: F401  (declares torch.ops.mindiesd.*)
+from .flash_attn import attention_forward, sparse_attention
 
-__all__ = ["attention_forward"]
+__all__ = ["attention_forward", "sparse_attention"]

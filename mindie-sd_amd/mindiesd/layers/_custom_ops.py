@@ -1,0 +1,199 @@
+"""``torch.ops.mindiesd.*`` operators of the attention path and their keyword wrappers.
+
+Schemas of ``rainfusionattention`` and ``block_sparse_attention`` are the reference's
+(csrc/plugin/register_ops.cpp:41-45, :62-67); the wrappers mirror mindiesd/layers/_custom_ops.py
+(:124-189, :330-390).  ``flash_attention_fwd`` is the dense kernel as an op."""
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import register_ops
+from ..utils.exception import ParametersInvalid
+
+register_ops.define_op(
+    "rainfusionattention",
+    "(Tensor query, Tensor key, Tensor value, Tensor select_idx, Tensor select_num_idx, int[] blockshape, "
+    "Tensor? attn_mask=None, int[]? actual_seq_qlen=None, int[]? actual_seq_kvlen=None, Tensor? block_table=None, "
+    "str q_input_layout='TND', str kv_input_layout='TND', int head_num=1, int mask_type=0, float scale=1.0, "
+    "int inner_precise=1, int block_size=0) -> (Tensor, Tensor)")
+register_ops.define_op(
+    "block_sparse_attention",
+    "(Tensor query, Tensor key, Tensor value, Tensor? block_sparse_mask=None, int[] block_shape=[128,128], "
+    "str q_input_layout='BNSD', str kv_input_layout='BNSD', int num_key_value_heads=1, float scale_value=1.0, "
+    "int inner_precise=0, int[]? actual_seq_lengths=None, int[]? actual_seq_lengths_kv=None, "
+    "int softmax_lse_flag=0) -> (Tensor, Tensor)")
+register_ops.define_op(
+    "flash_attention_fwd",
+    "(Tensor query, Tensor key, Tensor value, float scale_value=1.0, str input_layout='BNSD') -> (Tensor, Tensor)")
+
+
+def _tnd_as_bsnd(t, seq_lens, what):
+    """View a packed [T, N, D] tensor whose sequences all have one length as [B, S, N, D]."""
+    if t.dim() != 3:
+        raise RuntimeError(f"{what}: TND layout expects a 3-D tensor, got {t.dim()}-D")
+    if not seq_lens:
+        return t.unsqueeze(0)
+    if len(set(seq_lens)) != 1 or seq_lens[0] * len(seq_lens) != t.shape[0]:
+        raise RuntimeError(f"{what}: TND layout supports equal sequence lengths that sum to T only")
+    return t.reshape(len(seq_lens), seq_lens[0], t.shape[1], t.shape[2])
+
+
+def _check_lengths(actual, s, what):
+    if actual is not None and any(int(a) != s for a in actual):
+        raise RuntimeError(f"{what}: per-batch sequence lengths shorter than the tensor are not supported")
+
+
+@register_ops.register_device_impl("flash_attention_fwd")
+def _flash_attention_fwd_impl(query, key, value, scale_value=1.0, input_layout="BNSD"):
+    from .flash_attn.hip_flash_attn import flash_attention
+    if input_layout not in ("BNSD", "BSND"):
+        raise RuntimeError(f"flash_attention_fwd: input_layout only supports 'BNSD' and 'BSND', got {input_layout}")
+    return flash_attention(query, key, value, scale_value, input_layout, return_lse=True)
+
+
+@register_ops.register_mindie_fake_op("flash_attention_fwd")
+def _flash_attention_fwd_fake(query, key, value, scale_value=1.0, input_layout="BNSD"):
+    b, n, s = (query.shape[0], query.shape[1], query.shape[2]) if input_layout == "BNSD" else \
+        (query.shape[0], query.shape[2], query.shape[1])
+    return torch.empty_like(query), torch.empty((b, n, s), device=query.device, dtype=torch.float32)
+
+
+@register_ops.register_device_impl("block_sparse_attention")
+def _block_sparse_attention_impl(query, key, value, block_sparse_mask=None, block_shape=(128, 128),
+                                 q_input_layout="BNSD", kv_input_layout="BNSD", num_key_value_heads=1,
+                                 scale_value=1.0, inner_precise=0, actual_seq_lengths=None,
+                                 actual_seq_lengths_kv=None, softmax_lse_flag=0):
+    """csrc/plugin/block_sparse_attention.cpp:31-121: same argument checks (RuntimeError), callee
+    allocates ``(attention_out like query, softmax_lse fp32 [B,N,S,1] or [T,N,1])``; the lse is only
+    written when ``softmax_lse_flag != 0``."""
+    from .flash_attn import rainfusion as rf
+    if q_input_layout not in ("TND", "BNSD"):
+        raise RuntimeError(f"block_sparse_attention: q_input_layout only supports 'TND' and 'BNSD', got {q_input_layout}")
+    if kv_input_layout not in ("TND", "BNSD"):
+        raise RuntimeError(f"block_sparse_attention: kv_input_layout only supports 'TND' and 'BNSD', got {kv_input_layout}")
+    if q_input_layout != kv_input_layout:
+        raise RuntimeError("block_sparse_attention: q_input_layout and kv_input_layout must be consistent.")
+    if q_input_layout == "TND" and (actual_seq_lengths is None or actual_seq_lengths_kv is None):
+        raise RuntimeError("block_sparse_attention: actual_seq_lengths and actual_seq_lengths_kv are required "
+                           "for TND layout.")
+    if list(block_shape) != [128, 128]:
+        raise RuntimeError(f"block_sparse_attention: block_shape only supports [128, 128], got {list(block_shape)}")
+    if block_sparse_mask is None:
+        raise RuntimeError("block_sparse_attention: block_sparse_mask is required")
+    if q_input_layout == "TND":
+        q4 = _tnd_as_bsnd(query, list(actual_seq_lengths), "block_sparse_attention")
+        k4 = _tnd_as_bsnd(key, list(actual_seq_lengths_kv), "block_sparse_attention")
+        v4 = _tnd_as_bsnd(value, list(actual_seq_lengths_kv), "block_sparse_attention")
+        layout = "BSND"
+    else:
+        q4, k4, v4, layout = query, key, value, "BNSD"
+        _check_lengths(actual_seq_lengths, query.shape[2], "block_sparse_attention")
+        _check_lengths(actual_seq_lengths_kv, key.shape[2], "block_sparse_attention")
+    idx, cnt = rf.mask_to_lists(block_sparse_mask)
+    want_lse = softmax_lse_flag != 0
+    res = rf.block_sparse_attention_lists(q4, k4, v4, idx, cnt, scale_value, layout, return_lse=want_lse)
+    out, lse = res if want_lse else (res, None)
+    if q_input_layout == "TND":
+        out = out.reshape(query.shape)
+        lse_out = torch.empty((query.shape[0], query.shape[1], 1), dtype=torch.float32, device=query.device)
+        if want_lse:  # [B, N, S] -> [T, N, 1]
+            lse_out.copy_(lse.permute(0, 2, 1).reshape(query.shape[0], query.shape[1], 1))
+    else:
+        lse_out = lse.unsqueeze(-1) if want_lse else torch.empty(
+            (query.shape[0], query.shape[1], query.shape[2], 1), dtype=torch.float32, device=query.device)
+    return out, lse_out
+
+
+@register_ops.register_mindie_fake_op("block_sparse_attention")
+def block_sparse_attention_fake(query, key, value, block_sparse_mask=None, block_shape=None, q_input_layout="BNSD",
+                                kv_input_layout="BNSD", num_key_value_heads=1, scale_value=1.0, inner_precise=0,
+                                actual_seq_lengths=None, actual_seq_lengths_kv=None, softmax_lse_flag=0):
+    if q_input_layout == "TND":
+        lse_shape = [query.shape[0], query.shape[1], 1]
+    else:
+        lse_shape = [query.shape[0], query.shape[1], query.shape[2], 1]
+    return torch.empty_like(query), torch.empty(lse_shape, device=query.device, dtype=torch.float32)
+
+
+@register_ops.register_device_impl("rainfusionattention")
+def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blockshape, attn_mask=None,
+                              actual_seq_qlen=None, actual_seq_kvlen=None, block_table=None, q_input_layout="TND",
+                              kv_input_layout="TND", head_num=1, mask_type=0, scale=1.0, inner_precise=1,
+                              block_size=0):
+    """csrc/plugin/rainfusionattention.cpp:27-64.  ``select_idx`` [qb, N, kb] (-1 padded),
+    ``select_num_idx`` [qb, N]: one selection shared by every batch entry (the reference builds it
+    from batch 0, sparse_flash_attn_rf_v2.py:131-134).  Returns ``(out, softmax_lse)`` with the
+    reference's lse shape ``query.shape[:3]`` in the query dtype."""
+    from .flash_attn import rainfusion as rf
+    if q_input_layout not in ("TND", "BNSD"):
+        raise RuntimeError("q_input_layout only supports 'TND' and 'BNSD' now.")
+    if kv_input_layout not in ("TND", "BNSD"):
+        raise RuntimeError("kv_input_layout only supports 'TND' and 'BNSD' now.")
+    if q_input_layout != kv_input_layout:
+        raise RuntimeError("q_input_layout and kv_input_layout must be consistent.")
+    if list(blockshape) != [128, 128]:
+        raise RuntimeError(f"blockshape only supports [128, 128], got {list(blockshape)}")
+    if attn_mask is not None or block_table is not None or mask_type != 0 or block_size != 0:
+        raise RuntimeError("attn_mask / block_table / mask_type / block_size are not supported.")
+    if q_input_layout == "TND":
+        q4 = _tnd_as_bsnd(query, list(actual_seq_qlen) if actual_seq_qlen else None, "rainfusionattention")
+        k4 = _tnd_as_bsnd(key, list(actual_seq_kvlen) if actual_seq_kvlen else None, "rainfusionattention")
+        v4 = _tnd_as_bsnd(value, list(actual_seq_kvlen) if actual_seq_kvlen else None, "rainfusionattention")
+        layout = "BSND"
+        b, n = q4.shape[0], q4.shape[2]
+    else:
+        q4, k4, v4, layout = query, key, value, "BNSD"
+        b, n = query.shape[0], query.shape[1]
+    if select_idx.dim() != 3 or select_idx.shape[1] != n or tuple(select_num_idx.shape) != tuple(select_idx.shape[:2]):
+        raise RuntimeError("select_idx must be [q_blocks, N, kv_blocks] and select_num_idx [q_blocks, N]")
+    idx = select_idx.permute(1, 0, 2).to(torch.int32).unsqueeze(0).expand(b, -1, -1, -1).contiguous()
+    cnt = select_num_idx.permute(1, 0).to(torch.int32).unsqueeze(0).expand(b, -1, -1).contiguous()
+    out, lse = rf.block_sparse_attention_lists(q4, k4, v4, idx, cnt, scale, layout, return_lse=True)
+    if q_input_layout == "TND":
+        out = out.reshape(query.shape)
+        lse_out = torch.zeros(query.shape, dtype=query.dtype, device=query.device)
+        lse_out[:, :, 0] = lse.permute(0, 2, 1).reshape(query.shape[0], query.shape[1]).to(query.dtype)
+    else:
+        lse_out = lse.to(query.dtype)
+    return out, lse_out
+
+
+@register_ops.register_mindie_fake_op("rainfusionattention")
+def rain_fusion_attention_fake(query, key, value, select_idx, select_num_idx, blockshape, attn_mask=None,
+                               actual_seq_qlen=None, actual_seq_kvlen=None, block_table=None, q_input_layout="TND",
+                               kv_input_layout="TND", head_num=1, mask_type=0, scale=1.0, inner_precise=1,
+                               block_size=0):
+    lse = torch.empty([query.shape[0], query.shape[1], query.shape[2]], device=query.device, dtype=query.dtype)
+    return torch.empty_like(query), lse
+
+
+def rain_fusion_attention(query, key, value, select_idx, select_num_idx, blockshape: List[int],
+                          attn_mask: Optional[torch.Tensor] = None, actual_seq_qlen: Optional[List[int]] = None,
+                          actual_seq_kvlen: Optional[List[int]] = None, block_table: Optional[torch.Tensor] = None,
+                          q_input_layout: str = "TND", kv_input_layout: str = "TND", head_num: int = 1,
+                          mask_type: int = 0, scale: float = 1.0, inner_precise: int = 1,
+                          block_size: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    return torch.ops.mindiesd.rainfusionattention(
+        query=query, key=key, value=value, select_idx=select_idx, select_num_idx=select_num_idx,
+        blockshape=blockshape, attn_mask=attn_mask, actual_seq_qlen=actual_seq_qlen,
+        actual_seq_kvlen=actual_seq_kvlen, block_table=block_table, q_input_layout=q_input_layout,
+        kv_input_layout=kv_input_layout, head_num=head_num, mask_type=mask_type, scale=scale,
+        inner_precise=inner_precise, block_size=block_size)
+
+
+def block_sparse_attention(query, key, value, block_sparse_mask: Optional[torch.Tensor] = None,
+                           block_shape: List[int] = None, q_input_layout: str = "BNSD", kv_input_layout: str = "BNSD",
+                           num_key_value_heads: int = 1, scale_value: float = 1.0, inner_precise: int = 0,
+                           actual_seq_lengths: Optional[List[int]] = None,
+                           actual_seq_lengths_kv: Optional[List[int]] = None,
+                           softmax_lse_flag: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    kwargs = dict(query=query, key=key, value=value, block_sparse_mask=block_sparse_mask,
+                  block_shape=block_shape if block_shape is not None else [128, 128],
+                  q_input_layout=q_input_layout, kv_input_layout=kv_input_layout,
+                  num_key_value_heads=num_key_value_heads, scale_value=scale_value, inner_precise=inner_precise,
+                  softmax_lse_flag=softmax_lse_flag)
+    if actual_seq_lengths is not None:
+        kwargs["actual_seq_lengths"] = actual_seq_lengths
+    if actual_seq_lengths_kv is not None:
+        kwargs["actual_seq_lengths_kv"] = actual_seq_lengths_kv
+    return torch.ops.mindiesd.block_sparse_attention(**kwargs)

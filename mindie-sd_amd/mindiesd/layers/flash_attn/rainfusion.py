@@ -1,0 +1,349 @@
+"""RainFusion2.0 block-sparse attention on the MI355X.
+
+GPU counterparts of the reference's host pipeline
+(mindiesd/layers/flash_attn/sparse_flash_attn_rf_v2.py and sparse_flash_attn_rf_v3.py):
+window permutation and block mean pooling run as one HBM pass, the block mask (pooled scores,
+softmax, top-k threshold, forced text / first-frame blocks) as one kernel that also emits the
+compacted block lists the attention kernel walks, then the block-sparse flash-attention kernel and
+the inverse permutation.  Every function keeps the reference's signature and layouts.
+"""
+import math
+
+import torch
+
+from .hip_flash_attn import HEAD_DIM, _strides_bns
+from ... import _native
+from ...utils.exception import ParametersInvalid
+
+BLOCK = 128
+
+
+def _check_gpu16(t, what):
+    if not isinstance(t, torch.Tensor) or t.dim() != 4:
+        raise ParametersInvalid(f"{what} must be a 4-D torch.Tensor.")
+    if not t.is_cuda:
+        raise ParametersInvalid(f"{what} must live on the GPU, but is on {t.device}.")
+    if t.dtype not in _native.DTYPE_CODE:
+        raise ParametersInvalid(f"{what} must be bf16 or fp16, but got {t.dtype}.")
+    if t.shape[-1] != HEAD_DIM:
+        raise ParametersInvalid(f"{what} must have head_dim == {HEAD_DIM}, but got {t.shape[-1]}.")
+
+
+def _check_layout(input_layout):
+    if input_layout not in ("BSND", "BNSD"):
+        raise ParametersInvalid(f"The input_layout must in ['BSND', 'BNSD'], but got {input_layout}.")
+
+
+def _dims(t, layout):
+    """(B, N, S) of a 4-D tensor in ``layout``."""
+    return (t.shape[0], t.shape[1], t.shape[2]) if layout == "BNSD" else (t.shape[0], t.shape[2], t.shape[1])
+
+
+def _aligned(t):
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
+def _pool_strides(pool, layout):
+    """(batch, head, block) strides of a pooled tensor [X, N, NB, D] / [X, NB, N, D]."""
+    return _strides_bns(pool, layout)
+
+
+def _run_rearrange(srcs, dsts, pool, layout, grid, txt_len, inverse):
+    """Launch the permute(+pool) kernel on 1..3 same-shaped tensors.  ``grid`` = (t, h, w) or
+    (0, 0, 0) for the identity order.  ``pool`` is [len(srcs) * B, ...] in ``layout`` or None."""
+    x = srcs[0]
+    b, n, s = _dims(x, layout)
+    ptr = lambda lst, i: lst[i].data_ptr() if i < len(lst) and lst[i] is not None else None
+    d0 = dsts[0] if dsts and dsts[0] is not None else x
+    if pool is not None:
+        psb, psn, psblk = _pool_strides(pool, layout)
+        pst = b * pool.stride(0)
+    else:
+        pst = psb = psn = psblk = 0
+    with torch.cuda.device(x.device):
+        rc = _native.lib().mindiesd_rf_rearrange_pool(
+            ptr(srcs, 0), ptr(srcs, 1), ptr(srcs, 2), ptr(dsts, 0), ptr(dsts, 1), ptr(dsts, 2),
+            pool.data_ptr() if pool is not None else None, _native.DTYPE_CODE[x.dtype], b, n, s, x.shape[-1],
+            *_strides_bns(x, layout), *_strides_bns(d0, layout), pst, psb, psn, psblk,
+            int(grid[0]), int(grid[1]), int(grid[2]), int(txt_len), int(inverse), len(srcs),
+            _native.stream_ptr(x.device))
+    _native.check(rc, "mindiesd_rf_rearrange_pool")
+
+
+def _same_strides(ts):
+    return all(t.stride() == ts[0].stride() and t.shape == ts[0].shape for t in ts)
+
+
+def _check_grid(latent_shape, s_img):
+    t, h, w = (int(v) for v in latent_shape)
+    if t <= 0 or h < 8 or w < 8:
+        raise ParametersInvalid(f"latent_shape_q must be (t, h, w) with h >= 8 and w >= 8, but got {latent_shape}.")
+    if t * h * w != s_img:
+        raise ParametersInvalid(f"latent_shape_q {latent_shape} does not match the image sequence length {s_img}.")
+    return t, h, w
+
+
+# ------------------------------------------------------------------------------------------------
+# rf_v2.py:24-73
+# ------------------------------------------------------------------------------------------------
+def avgpool(input_tensor, pool_size=128, input_layout="BNSD"):
+    """Mean over consecutive 128-token blocks (a shorter tail block averages its own length)."""
+    _check_layout(input_layout)
+    _check_gpu16(input_tensor, "input_tensor")
+    if pool_size != BLOCK:
+        raise ParametersInvalid(f"pool_size only supports {BLOCK}, but got {pool_size}.")
+    x = _aligned(input_tensor)
+    b, n, s = _dims(x, input_layout)
+    nb = (s + BLOCK - 1) // BLOCK
+    shape = (b, n, nb, x.shape[-1]) if input_layout == "BNSD" else (b, nb, n, x.shape[-1])
+    pool = torch.empty(shape, dtype=x.dtype, device=x.device)
+    _run_rearrange([x], [None], pool, input_layout, (0, 0, 0), 0, 0)
+    return pool
+
+
+# ------------------------------------------------------------------------------------------------
+# rf_v2.py:137-289
+# ------------------------------------------------------------------------------------------------
+def rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k=None, input_layout="BNSD"):
+    """8x8-window token order (all frames if h and w are multiples of 8, else frames 1.. with the
+    remainder rows/columns appended per frame).  Only ``latent_shape_q`` is used, as in the reference."""
+    _check_layout(input_layout)
+    _check_gpu16(tensor, "tensor")
+    x = _aligned(tensor)
+    grid = _check_grid(latent_shape_q, _dims(x, input_layout)[2])
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _run_rearrange([x], [out], None, input_layout, grid, 0, 0)
+    return out
+
+
+def inv_rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k=None, input_layout="BNSD"):
+    _check_layout(input_layout)
+    _check_gpu16(tensor, "tensor")
+    x = _aligned(tensor)
+    grid = _check_grid(latent_shape_q, _dims(x, input_layout)[2])
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _run_rearrange([x], [out], None, input_layout, grid, 0, 1)
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# rf_v2.py:292-337 and rf_v3.py:100-118
+# ------------------------------------------------------------------------------------------------
+def _rearrange_qkv(query, key, value, text_len, latent_shape_q, input_layout, want_pool):
+    _check_layout(input_layout)
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        _check_gpu16(t, name)
+    if not (query.shape == key.shape == value.shape and query.dtype == key.dtype == value.dtype):
+        raise ParametersInvalid("RainFusion needs query, key and value of one shape and dtype "
+                                "(self-attention over the latent grid).")
+    q, k, v = _aligned(query), _aligned(key), _aligned(value)
+    if not _same_strides((q, k, v)):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    b, n, s = _dims(q, input_layout)
+    grid = _check_grid(latent_shape_q, s - text_len)
+    outs = [torch.empty(q.shape, dtype=q.dtype, device=q.device) for _ in range(3)]
+    pool = None
+    if want_pool:
+        nb = (s - text_len + BLOCK - 1) // BLOCK + (text_len + BLOCK - 1) // BLOCK
+        shape = (3 * b, n, nb, q.shape[-1]) if input_layout == "BNSD" else (3 * b, nb, n, q.shape[-1])
+        pool = torch.empty(shape, dtype=q.dtype, device=q.device)
+    _run_rearrange([q, k, v], outs, pool, input_layout, grid, text_len, 0)
+    return outs[0], outs[1], outs[2], pool
+
+
+def do_tensor_rearrange_pooling(query, key, value, text_len, pool_size, latent_shape_q, latent_shape_k,
+                                input_layout):
+    """Returns the permuted q, k, v ([image in window order | text]) and the pooled tensor
+    [3B, ...] (image blocks, then text blocks), all in ``input_layout``."""
+    if pool_size != BLOCK:
+        raise ParametersInvalid(f"pool_size only supports {BLOCK}, but got {pool_size}.")
+    return _rearrange_qkv(query, key, value, text_len, latent_shape_q, input_layout, True)
+
+
+def do_tensor_rearrange_only(q, k, v, txt_len, latent_shape_q, latent_shape_k, input_layout):
+    """Permutation without pooling, used when the block mask is cached (rf_v3.py:100-118)."""
+    return _rearrange_qkv(q, k, v, txt_len, latent_shape_q, input_layout, False)[:3]
+
+
+def do_tensor_inv_rearrange(tensor, text_len, latent_shape_q, latent_shape_k, input_layout):
+    """Undo the permutation and move the text tokens back to the front."""
+    _check_layout(input_layout)
+    _check_gpu16(tensor, "tensor")
+    x = _aligned(tensor)
+    grid = _check_grid(latent_shape_q, _dims(x, input_layout)[2] - text_len)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _run_rearrange([x], [out], None, input_layout, grid, text_len, 1)
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# rf_v2.py:76-134
+# ------------------------------------------------------------------------------------------------
+def get_mask_index(mask):
+    """Per row: ascending indices of the True entries, padded with -1; int64 [B, N, S, S]."""
+    if mask.dim() != 4 or not mask.is_cuda:
+        raise ParametersInvalid("mask must be a 4-D GPU tensor [B, N, S, S].")
+    b, n, qb, kb = mask.shape
+    m8 = mask.to(torch.int8).contiguous()
+    idx = torch.empty((b, n, qb, kb), dtype=torch.int32, device=mask.device)
+    cnt = torch.empty((b, n, qb), dtype=torch.int32, device=mask.device)
+    with torch.cuda.device(mask.device):
+        rc = _native.lib().mindiesd_mask_to_index(m8.data_ptr(), b * n, qb, kb, idx.data_ptr(), cnt.data_ptr(), kb,
+                                                  _native.stream_ptr(mask.device))
+    _native.check(rc, "mindiesd_mask_to_index")
+    return idx.to(torch.int64)
+
+
+def keep_len_of(cols, sparsity):
+    """Number of key blocks kept per row before forced blocks (rf_v2.py:112, same float expression)."""
+    return math.ceil(cols * (1 - sparsity))
+
+
+def _block_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout, protect_first_frame,
+                keep_diagonal, want_mask, want_lists, want_ref_lists):
+    _check_layout(input_layout)
+    _check_gpu16(qkv_pool, "qkv_pool")
+    if qkv_pool.shape[0] % 3 != 0:
+        raise ParametersInvalid("qkv_pool must stack the pooled query, key and value along dim 0.")
+    pool = _aligned(qkv_pool)
+    b = pool.shape[0] // 3
+    _, n, nb = _dims(pool, input_layout)
+    keep_len = keep_len_of(nb, sparsity)
+    if not 1 <= keep_len <= nb:
+        raise ParametersInvalid(f"sparsity must be in [0, 1), but got {sparsity}.")
+    txt_blocks = (txt_len + pool_size - 1) // pool_size
+    ff_blocks = 0
+    if protect_first_frame:
+        ff_blocks = min(nb, (int(latent_shape_q[1]) * int(latent_shape_q[2]) + pool_size - 1) // pool_size)
+    dev = pool.device
+    mask = torch.empty((b, n, nb, nb), dtype=torch.int8, device=dev) if want_mask else None
+    idx = torch.empty((b, n, nb, nb), dtype=torch.int32, device=dev) if want_lists else None
+    cnt = torch.empty((b, n, nb), dtype=torch.int32, device=dev) if want_lists else None
+    sel = torch.empty((nb, n, nb), dtype=torch.int64, device=dev) if want_ref_lists else None
+    sel_num = torch.empty((nb, n), dtype=torch.int64, device=dev) if want_ref_lists else None
+    qp, kp = pool[:b], pool[b:2 * b]
+    p = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(dev):
+        rc = _native.lib().mindiesd_rf_block_mask(
+            qp.data_ptr(), kp.data_ptr(), _native.DTYPE_CODE[pool.dtype], b, n, nb, pool.shape[-1],
+            *_pool_strides(qp, input_layout), float(scale), keep_len, txt_blocks, ff_blocks, int(bool(keep_diagonal)),
+            p(mask), p(idx), p(cnt), nb, p(sel), p(sel_num), _native.stream_ptr(dev))
+    _native.check(rc, "mindiesd_rf_block_mask")
+    return mask, idx, cnt, sel, sel_num
+
+
+def get_blockwise_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_shape_q, latent_shape_k, input_layout,
+                       return_binary=False, protect_first_frame=True, keep_diagonal=False):
+    """Block mask from pooled q/k: ``softmax(q_pool . k_pool * scale) >= k-th largest`` per row with
+    ``k = ceil(cols * (1 - sparsity))`` (ties keep extra blocks), text and first-frame rows/columns
+    forced.  Returns int8 [B, N, qb, kb] if ``return_binary`` else the reference's
+    ``(select_idx [qb, N, kb] int64 padded with -1, select_num_idx [qb, N])`` of batch 0.
+    ``keep_diagonal`` (not in the reference) also forces the diagonal blocks."""
+    if pool_size != BLOCK:
+        raise ParametersInvalid(f"pool_size only supports {BLOCK}, but got {pool_size}.")
+    mask, _, _, sel, sel_num = _block_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout,
+                                           protect_first_frame, keep_diagonal, return_binary, False, not return_binary)
+    if return_binary:
+        return mask
+    return sel, sel_num
+
+
+# ------------------------------------------------------------------------------------------------
+# block-sparse attention kernels (rf_v2.py:351-381, rf_v3.py:122-190)
+# ------------------------------------------------------------------------------------------------
+def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, layout="BNSD", return_lse=False):
+    """Attention of every 128-row query block over the key blocks listed for it.
+    ``blk_idx`` int32 [B, N, qb, stride] ascending block ids, ``blk_cnt`` int32 [B, N, qb].
+    A query block with an empty list yields zeros."""
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        _check_gpu16(t, name)
+    q, k, v = _aligned(query), _aligned(key), _aligned(value)
+    b, n, sq = _dims(q, layout)
+    _, nkv, skv = _dims(k, layout)
+    if k.shape != v.shape or k.shape[0] != b or n % nkv != 0 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ParametersInvalid("Inconsistent query/key/value shapes or dtypes.")
+    qb, kb = (sq + BLOCK - 1) // BLOCK, (skv + BLOCK - 1) // BLOCK
+    if (blk_idx.dtype != torch.int32 or blk_cnt.dtype != torch.int32 or tuple(blk_cnt.shape) != (b, n, qb)
+            or tuple(blk_idx.shape[:3]) != (b, n, qb) or not blk_idx.is_contiguous() or not blk_cnt.is_contiguous()):
+        raise ParametersInvalid(f"block lists must be contiguous int32 [B,N,{qb},stride] / [B,N,{qb}].")
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, n, sq), dtype=torch.float32, device=q.device) if return_lse else None
+    with torch.cuda.device(q.device):
+        rc = _native.lib().mindiesd_block_sparse_attention_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
+            _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1],
+            *_strides_bns(q, layout), *_strides_bns(k, layout), *_strides_bns(v, layout), *_strides_bns(out, layout),
+            float(scale), blk_idx.data_ptr(), blk_cnt.data_ptr(), blk_idx.shape[3], None,
+            _native.stream_ptr(q.device))
+    _native.check(rc, "mindiesd_block_sparse_attention_fwd")
+    return (out, lse) if return_lse else out
+
+
+def mask_to_lists(block_sparse_mask):
+    """int8/bool [B, N, qb, kb] (non-zero = attend) -> (blk_idx int32 [B,N,qb,kb], blk_cnt int32 [B,N,qb])."""
+    if block_sparse_mask.dim() != 4 or not block_sparse_mask.is_cuda:
+        raise ParametersInvalid("block_sparse_mask must be a 4-D GPU tensor [B, N, q_blocks, kv_blocks].")
+    m8 = block_sparse_mask.to(torch.int8).contiguous()
+    b, n, qb, kb = m8.shape
+    idx = torch.empty((b, n, qb, kb), dtype=torch.int32, device=m8.device)
+    cnt = torch.empty((b, n, qb), dtype=torch.int32, device=m8.device)
+    with torch.cuda.device(m8.device):
+        rc = _native.lib().mindiesd_mask_to_index(m8.data_ptr(), b * n, qb, kb, idx.data_ptr(), cnt.data_ptr(), kb,
+                                                  _native.stream_ptr(m8.device))
+    _native.check(rc, "mindiesd_mask_to_index")
+    return idx, cnt
+
+
+def rain_fusion_attention(query, key, value, scale=None, head_num=None, input_layout="TND", select_idx=None,
+                          select_num_idx=None, blockshape=None, actual_seq_lengths=None, actual_seq_lengths_kv=None,
+                          inner_precise=0):
+    """Index-list driven sparse attention (rf_v2.py:351-381).  ``select_idx`` [qb, N, kb] int64 (-1
+    padded), ``select_num_idx`` [qb, N]; layouts 'TND' (one sequence) or 'BNSD'."""
+    from .. import _custom_ops as ops
+    out, _ = ops.rain_fusion_attention(
+        query, key, value, select_idx, select_num_idx, blockshape if blockshape is not None else [BLOCK, BLOCK],
+        attn_mask=None, actual_seq_qlen=actual_seq_lengths, actual_seq_kvlen=actual_seq_lengths_kv, block_table=None,
+        q_input_layout=input_layout, kv_input_layout=input_layout, head_num=head_num if head_num is not None else 1,
+        mask_type=0, scale=scale if scale is not None else query.shape[-1] ** -0.5, inner_precise=inner_precise,
+        block_size=0)
+    return out
+
+
+def rain_fusion_attention_v3(query, key, value, block_sparse_mask, scale=None, head_num=None, num_key_value_heads=None,
+                             input_layout="BNSD", actual_seq_lengths=None, actual_seq_lengths_kv=None, sparse_size=128,
+                             inner_precise=4):
+    """Mask driven sparse attention (rf_v3.py:122-190): int8 mask [B, N, qb, kb], 1 = attend.  BSND
+    inputs run in place (the reference copies them to BNSD first)."""
+    if scale is None:
+        scale = query.shape[-1] ** -0.5
+    _check_layout(input_layout)
+    if sparse_size != BLOCK:
+        raise ParametersInvalid(f"sparse_size only supports {BLOCK}, but got {sparse_size}.")
+    idx, cnt = mask_to_lists(block_sparse_mask)
+    return block_sparse_attention_lists(query, key, value, idx, cnt, scale, input_layout)
+
+
+def bsa_sparse_attention_v3(q, k, v, latent_shape_q, latent_shape_k=None, txt_len=0, pool_size=128, sparsity=0.5,
+                            input_layout="BSND", head_num=None, num_key_value_heads=None, scale=None, inner_precise=4,
+                            cached_mask=None, protect_first_frame=True, keep_diagonal=False):
+    """End-to-end rf_v3 sparse attention (rf_v3.py:193-295): permute(+pool) -> mask -> block-sparse
+    attention -> inverse permute.  Returns ``(out, mask)``; pass the mask back as ``cached_mask`` on
+    later diffusion steps to skip pooling and mask generation."""
+    if latent_shape_k is None:
+        latent_shape_k = latent_shape_q
+    if scale is None:
+        scale = float(q.shape[-1]) ** -0.5
+    if pool_size != BLOCK:
+        raise ParametersInvalid(f"pool_size only supports {BLOCK}, but got {pool_size}.")
+    if cached_mask is None:
+        q_, k_, v_, pool = _rearrange_qkv(q, k, v, txt_len, latent_shape_q, input_layout, True)
+        new_mask, idx, cnt, _, _ = _block_mask(pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout,
+                                               protect_first_frame, keep_diagonal, True, True, False)
+    else:
+        q_, k_, v_, _ = _rearrange_qkv(q, k, v, txt_len, latent_shape_q, input_layout, False)
+        new_mask = cached_mask
+        idx, cnt = mask_to_lists(cached_mask)
+    out = block_sparse_attention_lists(q_, k_, v_, idx, cnt, scale, input_layout)
+    out = do_tensor_inv_rearrange(out, txt_len, latent_shape_q, latent_shape_k, input_layout)
+    return out, new_mask

@@ -1,0 +1,2 @@
+"""Import-path alias: the reference keeps these functions in sparse_flash_attn_rf_v3.py."""
+from .rainfusion import (do_tensor_rearrange_only, rain_fusion_attention_v3, bsa_sparse_attention_v3)  # noqa: F401

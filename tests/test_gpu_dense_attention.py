@@ -1,0 +1,137 @@
+"""GPU parity: the HIP flash-attention kernel behind attention_forward vs the CPU oracle
+(restatement of the reference's attention_math).  Tolerance (bf16): max-abs <= 2e-2 and
+cosine >= 0.9999; the reference's own fused-vs-fallback rule (data_compare) is checked as well."""
+import pytest
+import torch
+
+from oracle.attention import attention_math, attention_math_rows, cosine, data_compare
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+MIN_COS = 0.9999
+
+
+def _qkv(shape, seed, dtype=torch.bfloat16, mul=1.0, kv_shape=None):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(shape, generator=g) * mul).to(dtype)
+    k = (torch.randn(kv_shape or shape, generator=g) * mul).to(dtype)
+    v = (torch.randn(kv_shape or shape, generator=g) * mul).to(dtype)
+    return q, k, v
+
+
+def _check(out, ref, max_abs=MAX_ABS, min_cos=MIN_COS):
+    err = (out.float() - ref.float()).abs().max().item()
+    cos = cosine(out, ref)
+    assert err <= max_abs, f"max-abs {err}"
+    assert cos >= min_cos, f"cosine {cos}"
+
+
+@pytest.mark.parametrize("head_first", [True, False])
+@pytest.mark.parametrize("s", [1, 31, 128, 300, 1024, 1153])
+def test_small_shapes_both_layouts(cuda, head_first, s):
+    import mindiesd
+    shape = (2, 3, s, 128) if head_first else (2, s, 3, 128)
+    q, k, v = _qkv(shape, seed=s)
+    ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=head_first)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=head_first)
+    assert out.shape == q.shape and out.dtype == q.dtype
+    _check(out.cpu(), ref)
+
+
+def test_config1_full(cuda):
+    """B1 N12 S4096 D128 bf16 N(0,1), scale 1/sqrt(128): oracle evaluated whole."""
+    import mindiesd
+    q, k, v = _qkv((1, 12, 4096, 128), seed=1)
+    ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=True)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
+    _check(out, ref)
+    assert data_compare(out, ref, rel=4e-3), "reference's data_compare rule (threshold widened to one bf16 ulp)"
+
+
+def test_fp16(cuda):
+    import mindiesd
+    q, k, v = _qkv((1, 777, 4, 128), seed=5, dtype=torch.float16)
+    ref = attention_math(q, k, v, None, 0.11, head_first=False)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), scale=0.11).cpu()
+    _check(out, ref, max_abs=2e-3, min_cos=0.99999)
+    assert data_compare(out, ref), "reference's data_compare rule"
+
+
+def test_cross_attention_and_gqa(cuda):
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    q, k, v = _qkv((1, 8, 500, 128), seed=7, kv_shape=(1, 2, 1300, 128))
+    ref = attention_math(q, k.repeat_interleave(4, dim=1), v.repeat_interleave(4, dim=1), None, 128 ** -0.5, True)
+    out, lse = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", return_lse=True)
+    _check(out.cpu(), ref)
+    s = (q.float() @ k.repeat_interleave(4, dim=1).float().transpose(-1, -2)) * 128 ** -0.5
+    assert (lse.cpu() - torch.logsumexp(s, dim=-1)).abs().max() < 1e-4
+
+
+def test_strided_views_run_in_place(cuda):
+    """BSND tensors viewed as BNSD (and the reverse) must give the same result without a copy."""
+    import mindiesd
+    q, k, v = _qkv((1, 640, 5, 128), seed=9)
+    qc, kc, vc = q.to(cuda), k.to(cuda), v.to(cuda)
+    a = mindiesd.attention_forward(qc, kc, vc, head_first=False)
+    b = mindiesd.attention_forward(qc.transpose(1, 2), kc.transpose(1, 2), vc.transpose(1, 2), head_first=True)
+    assert torch.equal(a, b.transpose(1, 2))
+    for mode in ("static", "manual"):
+        c = mindiesd.attention_forward(qc, kc, vc, opt_mode=mode, op_type="ascend_laser_attention", layout="BSH")
+        assert torch.equal(a, c)
+
+
+def test_rising_row_maxima_vs_fp64(cuda):
+    """Late keys raise the row maxima far above what the first tiles saw, so the lazily updated
+    softmax reference maximum has to move several times.  Checked against an fp64 evaluation: in
+    this regime the bf16-rounded scores of the reference's unfused path are themselves too coarse
+    to serve as the yardstick."""
+    import mindiesd
+    from oracle.attention import attention_fp64
+    q, k, v = _qkv((1, 2, 2048, 128), seed=11, mul=1.5)
+    k[:, :, 700:1400] *= 2.0
+    k[:, :, 1400:] *= 3.0
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
+    for n in range(2):
+        ref = attention_fp64(q[0, n], k[0, n], v[0, n], 128 ** -0.5)
+        _check(out[0, n], ref, max_abs=5e-2)
+
+
+def test_config2_head_subset(cuda):
+    """Wan2.1-1.3B shape (S=32760): full GPU run, oracle on a row sample of two heads."""
+    import mindiesd
+    q, k, v = _qkv((1, 12, 32760, 128), seed=2, mul=0.5)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
+    for head in (0, 11):
+        for rows in (slice(0, 512), slice(32248, 32760)):
+            ref = attention_math_rows(q[:, head:head + 1], k[:, head:head + 1], v[:, head:head + 1], 128 ** -0.5,
+                                      row_chunk=512, q_rows=rows)
+            _check(out[:, head:head + 1, rows], ref)
+
+
+def test_unfused_path_matches_oracle(cuda):
+    import mindiesd
+    q, k, v = _qkv((1, 200, 2, 128), seed=13)
+    mask = torch.rand(200, 200) > 0.3
+    mask[:, 0] = True
+    ref = attention_math(q, k, v, mask, 0.09, head_first=False)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=mask.to(cuda), scale=0.09, fused=False)
+    _check(out.cpu(), ref)
+
+
+def test_errors(cuda):
+    import mindiesd
+    from mindiesd import ParametersInvalid
+    q = torch.randn(1, 64, 2, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q, q, q, opt_mode="fastest")
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q, q, q, scale=1)
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q[0], q, q)
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q.float(), q.float(), q.float())
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q[..., :64], q[..., :64], q[..., :64])
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward(q, q, q, opt_mode="manual", op_type="nope")
