@@ -1,0 +1,254 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+Prints ONE JSON line.  A step is one dense bf16 flash-attention forward at the Wan2.1-14B 720p
+shape (B=1, N=40, S=75600 = 21x45x80 latent grid, D=128, non-causal, scale 1/sqrt(128)) on synthetic
+N(0,1)*0.5 inputs already resident in HBM; ``value`` is the achieved TFLOP/s (4*N*S^2*D flops per
+step), which for a dense kernel equals the dense-equivalent figure.  ``roofline`` prices the same
+kernel against the bf16 dense MFMA peak, from HIP-event timings of the launches on the stream they
+run on.  ``extras`` carries the other workloads of the path (dense at the Wan2.1-1.3B shape,
+RainFusion block-sparse attention with and without mask generation, and - when built - FP8
+attention and the MXFP8 GEMM+SwiGLU).  ``cpu_baseline`` times the CPU oracle (a restatement of the
+reference's unfused torch path) on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mindie-sd_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+PEAK_HBM_GBS = 8000.0
+
+# workloads (BASELINE.json configs)
+CFG_14B_720P = dict(B=1, N=40, S=75600, D=128, grid=(21, 45, 80))
+CFG_1P3B = dict(B=1, N=12, S=32760, D=128, grid=(21, 30, 52))
+CFG_14B_480P = dict(B=1, N=40, S=32760, D=128, grid=(21, 30, 52))
+CFG_PARITY = dict(B=1, N=12, S=4096, D=128)
+CFG_FFN = dict(M=32760, K=5120, N=13824)
+
+
+def attn_flops(cfg):
+    return 4.0 * cfg["B"] * cfg["N"] * cfg["S"] * cfg["S"] * cfg["D"]
+
+
+# ---- synthetic inputs (seeded; generated on the device they are used on) ---------------------------
+def dense_inputs(cfg, device, seed=0, mul=0.5, dtype=None):
+    """q, k, v = mul * N(0,1), BNSD."""
+    import torch
+    dtype = dtype or torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(seed)
+    shape = (cfg["B"], cfg["N"], cfg["S"], cfg["D"])
+    return tuple((torch.randn(shape, generator=g, device=device, dtype=torch.float32) * mul).to(dtype)
+                 for _ in range(3))
+
+
+def _gauss_kernel(sigma, device):
+    import torch
+    r = int(math.ceil(3 * sigma))
+    x = torch.arange(-r, r + 1, device=device, dtype=torch.float32)
+    k = torch.exp(-0.5 * (x / sigma) ** 2)
+    return k / k.sum()
+
+
+def smooth_field_inputs(cfg, device, seed=0, sigma=2.0, noise=0.3, heads=None, dtype=None):
+    """q, k, v (BNSD, tokens flattened T-H-W): per (head, channel) an N(0,1) field on the latent grid,
+    Gaussian filtered with sigma tokens along T, H and W (separable, zero padded), renormalised to
+    unit variance per head, plus ``noise`` * N(0,1).  Block scores are therefore structured."""
+    import torch
+    import torch.nn.functional as F
+    dtype = dtype or torch.bfloat16
+    t, h, w = cfg["grid"]
+    n, d = (cfg["N"] if heads is None else heads), cfg["D"]
+    g = torch.Generator(device=device).manual_seed(seed)
+    kern = _gauss_kernel(sigma, device)
+    r = kern.numel() // 2
+    outs = []
+    for _ in range(3):
+        heads_out = []
+        for _n in range(n):
+            f = torch.randn((d, 1, t, h, w), generator=g, device=device)
+            f = F.conv3d(f, kern.view(1, 1, -1, 1, 1), padding=(r, 0, 0))
+            f = F.conv3d(f, kern.view(1, 1, 1, -1, 1), padding=(0, r, 0))
+            f = F.conv3d(f, kern.view(1, 1, 1, 1, -1), padding=(0, 0, r))
+            f = f / f.std()
+            f = f + noise * torch.randn(f.shape, generator=g, device=device)
+            heads_out.append(f.reshape(d, t * h * w).t().to(dtype))
+        outs.append(torch.stack(heads_out, 0).unsqueeze(0).contiguous())
+    return tuple(outs)
+
+
+# ---- timing -----------------------------------------------------------------------------------------
+def time_steps(fn, steps, warmup):
+    """Per-step durations in ms from HIP events on the current stream (the stream the kernels are
+    launched on), plus the wall-clock total of the timed region."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    evs[0].record()
+    for i in range(steps):
+        fn()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)], wall_ms
+
+
+def median(xs):
+    s = sorted(xs)
+    return s[len(s) // 2] if len(s) % 2 else 0.5 * (s[len(s) // 2 - 1] + s[len(s) // 2])
+
+
+# ---- CPU baseline -------------------------------------------------------------------------------------
+def cpu_baseline_dense(cfg, target_s=15.0):
+    """The oracle's attention_math (the reference's unfused torch path restated) on one head and a
+    sample of query rows against the full key/value sequence of the benchmark shape; throughput in
+    TFLOP/s over the sample."""
+    import torch
+    from oracle.attention import attention_math_rows
+    g = torch.Generator().manual_seed(0)
+    s, d = cfg["S"], cfg["D"]
+    k = (torch.randn(1, 1, s, d, generator=g) * 0.5).to(torch.bfloat16)
+    v = (torch.randn(1, 1, s, d, generator=g) * 0.5).to(torch.bfloat16)
+    rows = 256
+    q = (torch.randn(1, 1, rows, d, generator=g) * 0.5).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    attention_math_rows(q, k, v, d ** -0.5, row_chunk=256)
+    probe = time.perf_counter() - t0
+    rows = int(min(s, max(256, 256 * round(target_s / max(probe, 1e-3)))))
+    rows = min(rows, 8192)
+    q = (torch.randn(1, 1, rows, d, generator=g) * 0.5).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    attention_math_rows(q, k, v, d ** -0.5, row_chunk=256)
+    dt = time.perf_counter() - t0
+    flops = 4.0 * rows * s * d
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle attention_math, 1 head, {rows} query rows x {s} keys of the benchmark shape, "
+                  f"{dt:.1f} s on {os.cpu_count()} visible CPUs (torch threads {torch.get_num_threads()})",
+    }
+
+
+# ---- extras ---------------------------------------------------------------------------------------------
+def extra_dense_1p3b(device, steps, warmup):
+    import mindiesd
+    q, k, v = dense_inputs(CFG_1P3B, device, seed=2)
+    ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)
+    m = median(ms)
+    return {"workload": "dense bf16 B1 N12 S32760 D128", "ms": m, "tflops": attn_flops(CFG_1P3B) / m / 1e9,
+            "frac_of_bf16_peak": attn_flops(CFG_1P3B) / m / 1e9 / PEAK_BF16_TFLOPS}
+
+
+def extra_sparse(device, steps, warmup, dense_ms):
+    """RainFusion block-sparse attention at the 14B 720p shape: top 25 % of key blocks per query
+    block + first-frame blocks + diagonal.  Reported with the whole pipeline (permute + pool + mask +
+    attention + inverse permute) and with a cached mask (permute + attention + inverse permute)."""
+    import torch
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    cfg = CFG_14B_720P
+    q, k, v = smooth_field_inputs(cfg, device, seed=3)
+    args = dict(latent_shape_q=cfg["grid"], sparsity=0.75, input_layout="BNSD", keep_diagonal=True)
+    out, mask = rf.bsa_sparse_attention_v3(q, k, v, **args)
+    density = float(mask.float().mean())
+    full_ms, _ = time_steps(lambda: rf.bsa_sparse_attention_v3(q, k, v, **args), steps, warmup)
+    cached_ms, _ = time_steps(lambda: rf.bsa_sparse_attention_v3(q, k, v, cached_mask=mask, **args), steps, warmup)
+    # attention kernel alone on already permuted tensors and prebuilt lists
+    q_, k_, v_, pool = rf.do_tensor_rearrange_pooling(q, k, v, 0, 128, cfg["grid"], cfg["grid"], "BNSD")
+    idx, cnt = rf.mask_to_lists(mask)
+    kern_ms, _ = time_steps(lambda: rf.block_sparse_attention_lists(q_, k_, v_, idx, cnt, cfg["D"] ** -0.5, "BNSD"),
+                            steps, warmup)
+    mask_ms, _ = time_steps(lambda: rf.get_blockwise_mask(pool, 0, 0.75, cfg["D"] ** -0.5, 128, cfg["grid"],
+                                                          cfg["grid"], "BNSD", return_binary=True,
+                                                          keep_diagonal=True), steps, warmup)
+    perm_ms, _ = time_steps(lambda: rf.do_tensor_rearrange_pooling(q, k, v, 0, 128, cfg["grid"], cfg["grid"], "BNSD"),
+                            steps, warmup)
+    del out
+    torch.cuda.empty_cache()
+    f = attn_flops(cfg)
+    fm, cm, km = median(full_ms), median(cached_ms), median(kern_ms)
+    return {
+        "workload": "RainFusion rf_v3 B1 N40 S75600 D128, sparsity 0.75 + first frame + diagonal, smooth-field inputs",
+        "mask_density": density,
+        "pipeline_ms": fm, "pipeline_dense_equiv_tflops": f / fm / 1e9, "speedup_vs_dense": dense_ms / fm,
+        "cached_mask_ms": cm, "cached_mask_speedup_vs_dense": dense_ms / cm,
+        "attention_kernel_ms": km, "attention_kernel_tflops_actual": f * density / km / 1e9,
+        "attention_kernel_speedup_vs_dense": dense_ms / km,
+        "permute_pool_ms": median(perm_ms), "permute_pool_gbs": 6 * 774.144e6 / median(perm_ms) / 1e6,
+        "mask_ms": median(mask_ms),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one GPU's share of the attention path on ONE MI355X; "
+              "--gpus must be 1 (no collectives or sharding are part of it).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mindiesd
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    cfg = CFG_14B_720P
+    q, k, v = dense_inputs(cfg, device, seed=1)
+    step = lambda: mindiesd.attention_forward(q, k, v, head_first=True)
+    ms, wall_ms = time_steps(step, args.steps, args.warmup)
+    del q, k, v
+    torch.cuda.empty_cache()
+    ms_per_step = wall_ms / args.steps          # whole-job figure: wall clock of the timed region
+    kernel_ms = sum(ms) / len(ms)               # average launch duration from HIP events
+    flops = attn_flops(cfg)
+    value = flops / ms_per_step / 1e9
+    achieved = flops / kernel_ms / 1e9
+
+    result = {
+        "metric": "attn fwd TFLOPS (dense-equiv) + ms at Wan2.1-14B 720p shape; % of MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "dense bf16 flash-attention forward, B=1 N=40 S=75600 (21x45x80) D=128, non-causal, "
+                               "BNSD, q/k/v = 0.5*N(0,1) seeded"},
+        "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "fa_fwd_kernel<bf16, 8 waves x 32 rows, 128-key tiles>",
+                     "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms},
+    }
+    if not args.no_extras:
+        extras = {}
+        for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
+                         ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms))):
+            try:
+                extras[name] = fn()
+            except Exception as e:  # an extra must never cost the main line
+                extras[name] = {"error": f"{type(e).__name__}: {e}"}
+        result["extras"] = extras
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_dense(cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

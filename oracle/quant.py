@@ -1,0 +1,153 @@
+"""Oracle: FP8 / MXFP8 quantisation, FP8 attention and the MXFP8 GEMM+SwiGLU on the CPU
+(test infrastructure only).
+
+PARITY UNPINNED against the reference: the reference hands these steps to closed vendor ops
+(``torch_npu.npu_dynamic_block_quant`` mindiesd/layers/quant/block_quant.py:43-46,
+``npu_fused_infer_attention_score_v2`` mindiesd/quantization/layer.py:304-316,
+``npu_dynamic_mx_quant`` / ``npu_quant_matmul`` layer.py:338-361) and mocks them in its own tests
+(tests/quantization/test_layer.py:40-54), so there is no reference arithmetic to compare with.
+The functions below follow the published formats instead and are pinned against those:
+
+* OCP FP8 E4M3 ("e4m3fn": bias 7, 3 mantissa bits, max 448, no infinities), round to nearest even,
+  saturating -- ``e4m3_round`` is a bit-level implementation checked against all 256 codes and
+  against torch's ``float8_e4m3fn`` casts.
+* block scaling: ``scale = amax / 448`` in fp32 per block, ``q = e4m3(x / scale)`` (an all-zero
+  block gets scale 1), dequantisation ``x ~ q * scale``.
+* OCP Microscaling (MX) v1.0, MXFP8 E4M3: blocks of 32 along K share an E8M0 scale
+  ``2^(floor(log2(amax)) - 8)`` (8 = exponent of the largest E4M3 normal), elements are
+  ``e4m3(x / scale)`` saturated to +-448.
+"""
+import math
+
+import numpy as np
+import torch
+
+E4M3_MAX = 448.0
+
+
+# ---- E4M3 ---------------------------------------------------------------------------------------------
+def e4m3_decode(codes):
+    """uint8 codes -> float32 (0x7f / 0xff are NaN)."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.int32)
+    sign = np.where(c & 0x80, -1.0, 1.0)
+    e = (c >> 3) & 0xF
+    m = c & 0x7
+    val = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e.astype(np.float64) - 7))
+    val = np.where((e == 15) & (m == 7), np.nan, val)
+    return (sign * val).astype(np.float32)
+
+
+def e4m3_encode(x):
+    """float32 -> nearest E4M3 code, ties to even, magnitudes above 448 saturate to +-448."""
+    x = np.asarray(x, dtype=np.float32)
+    a = np.minimum(np.abs(x).astype(np.float64), E4M3_MAX)
+    # exponent of the grid: normals have 3 mantissa bits, subnormals a fixed step of 2^-9
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -6)))
+    step = np.exp2(e - 3)
+    q = np.rint(a / step) * step          # np.rint rounds half to even
+    q = np.minimum(q, E4M3_MAX)
+    e2 = np.floor(np.log2(np.maximum(q, 2.0 ** -6)))
+    mant = np.where(q < 2.0 ** -6, q / 2.0 ** -9, (q / np.exp2(e2) - 1.0) * 8.0)
+    expo = np.where(q < 2.0 ** -6, 0, e2 + 7)
+    code = (expo.astype(np.int32) << 3) | np.rint(mant).astype(np.int32)
+    code = np.where(np.signbit(x), code | 0x80, code)
+    return code.astype(np.uint8)
+
+
+def e4m3_round(x):
+    """float32 -> float32 value of the nearest E4M3 number (RNE, saturating)."""
+    return e4m3_decode(e4m3_encode(x))
+
+
+# ---- block quantisation of attention operands ----------------------------------------------------------
+def dynamic_block_quant(x, row_block=128, col_block=128):
+    """[..., S, D] -> (codes uint8 same shape, scale fp32 [..., ceil(S/row_block), ceil(D/col_block)]).
+    One scale per (row_block tokens x col_block channels) tile: scale = amax/448, q = e4m3(x/scale)."""
+    xf = x.float().numpy()
+    s, d = xf.shape[-2:]
+    nb_r, nb_c = math.ceil(s / row_block), math.ceil(d / col_block)
+    codes = np.zeros(xf.shape, dtype=np.uint8)
+    scale = np.ones(xf.shape[:-2] + (nb_r, nb_c), dtype=np.float32)
+    for i in range(nb_r):
+        for j in range(nb_c):
+            rs, cs = slice(i * row_block, (i + 1) * row_block), slice(j * col_block, (j + 1) * col_block)
+            blk = xf[..., rs, cs]
+            amax = np.abs(blk).max(axis=(-1, -2)).astype(np.float32)
+            sc = np.where(amax > 0, amax / np.float32(E4M3_MAX), np.float32(1.0)).astype(np.float32)
+            scale[..., i, j] = sc
+            codes[..., rs, cs] = e4m3_encode(blk / sc[..., None, None])
+    return torch.from_numpy(codes), torch.from_numpy(scale)
+
+
+def dequant_block(codes, scale, row_block=128, col_block=128):
+    q = torch.from_numpy(e4m3_decode(codes.numpy()))
+    s, d = q.shape[-2:]
+    sc = scale.repeat_interleave(row_block, dim=-2)[..., :s, :].repeat_interleave(col_block, dim=-1)[..., :d]
+    return q * sc
+
+
+def per_channel_quant(v):
+    """[..., S, D] -> (codes, scale [..., D]): one scale per channel over the whole sequence."""
+    vf = v.float().numpy()
+    amax = np.abs(vf).max(axis=-2).astype(np.float32)
+    sc = np.where(amax > 0, amax / np.float32(E4M3_MAX), np.float32(1.0)).astype(np.float32)
+    return torch.from_numpy(e4m3_encode(vf / sc[..., None, :])), torch.from_numpy(sc)
+
+
+def fp8_attention(query, key, value, scale=None):
+    """FP8 attention of the Wan2.1-14B 480p workload, BNSD: Q and K quantised per (head, 128-token
+    block) over all channels, V per (head, channel); everything is dequantised and run through plain
+    softmax(scale QK^T)V in fp32; bf16-typed output.  (The quantise -> dequantise path: the GPU kernel
+    additionally re-quantises the probabilities per tile, which this oracle does not model; the
+    stated tolerance, cosine >= 0.999, covers it.)"""
+    d = query.shape[-1]
+    if scale is None:
+        scale = d ** -0.5
+    qc, qs = dynamic_block_quant(query, 128, d)
+    kc, ks = dynamic_block_quant(key, 128, d)
+    vc, vs = per_channel_quant(value)
+    qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, 128, d)
+    vd = torch.from_numpy(e4m3_decode(vc.numpy())) * vs[..., None, :]
+    out = torch.empty(query.shape, dtype=torch.float32)
+    for r0 in range(0, query.shape[-2], 2048):
+        s = (qd[..., r0:r0 + 2048, :] @ kd.transpose(-1, -2)) * scale
+        out[..., r0:r0 + 2048, :] = torch.softmax(s, dim=-1) @ vd
+    return out.to(query.dtype)
+
+
+# ---- MX (microscaling) ----------------------------------------------------------------------------------
+def mx_quant(x, block=32):
+    """[M, K] -> (codes uint8 [M, K], e8m0 uint8 [M, K/block]); K must be a multiple of ``block``."""
+    xf = x.float().numpy()
+    m, k = xf.shape
+    assert k % block == 0
+    blk = xf.reshape(m, k // block, block)
+    amax = np.abs(blk).max(axis=-1)
+    _, ex = np.frexp(amax)                      # amax = f * 2^ex with f in [0.5, 1)  ->  floor(log2) = ex - 1
+    shared = np.where(amax > 0, ex - 1 - 8, -127)
+    shared = np.clip(shared, -127, 127).astype(np.int32)
+    codes = e4m3_encode(blk / np.exp2(shared.astype(np.float64))[..., None].astype(np.float32)).reshape(m, k)
+    return torch.from_numpy(codes), torch.from_numpy((shared + 127).astype(np.uint8))
+
+
+def mx_dequant(codes, e8m0, block=32):
+    q = e4m3_decode(codes.numpy()).astype(np.float64)
+    sc = np.exp2(e8m0.numpy().astype(np.float64) - 127)
+    return torch.from_numpy(q * np.repeat(sc, block, axis=-1))
+
+
+def mxfp8_gemm(x, w, bias=None):
+    """x [M, K], w [N, K] (both any float dtype) -> fp64 [M, N]: MX-quantise both along K,
+    dequantise, multiply exactly."""
+    xd = mx_dequant(*mx_quant(x))
+    wd = mx_dequant(*mx_quant(w))
+    out = xd @ wd.t()
+    return out if bias is None else out + bias.double()
+
+
+def mxfp8_gemm_swiglu(x, w, out_dtype=torch.bfloat16):
+    """w = [gate rows | up rows] ([2F, K]); returns silu(x w_gate^T) * (x w_up^T) as ``out_dtype`` [M, F]."""
+    y = mxfp8_gemm(x, w)
+    f = w.shape[0] // 2
+    gate, up = y[:, :f], y[:, f:]
+    return (gate / (1.0 + torch.exp(-gate)) * up).to(out_dtype)

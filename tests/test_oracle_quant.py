@@ -1,0 +1,104 @@
+"""Pins the quantisation oracle against the published formats: OCP FP8 E4M3 (all 256 codes, torch's
+own float8_e4m3fn casts, rounding ties, saturation) and OCP MX (power-of-two shared scales, element
+range), plus closed-form properties of the block scales and of the dequantised products."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+
+
+def test_e4m3_all_codes_round_trip_and_match_torch():
+    codes = np.arange(256, dtype=np.uint8)
+    vals = oq.e4m3_decode(codes)
+    tv = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    finite = ~np.isnan(tv)
+    assert np.isnan(vals[~finite]).all() and (~finite).sum() == 2          # 0x7f and 0xff only
+    assert np.array_equal(vals[finite], tv[finite])
+    assert vals[0x7e] == 448.0 and vals[0x08] == 2.0 ** -6 and vals[0x01] == 2.0 ** -9
+    back = oq.e4m3_encode(vals[finite])
+    keep = codes[finite]
+    assert np.array_equal(back[keep != 0x80], keep[keep != 0x80])           # -0 encodes as 0x80 too
+    assert back[keep == 0x80][0] == 0x80
+
+
+def test_e4m3_rounding_matches_torch_cast_and_saturates():
+    g = torch.Generator().manual_seed(0)
+    x = torch.cat([torch.randn(20000, generator=g) * s for s in (1e-3, 0.05, 1.0, 30.0, 200.0)])
+    x = x.clamp(-448, 448)
+    want = x.to(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(oq.e4m3_round(x.numpy()), want)
+    # ties go to the even mantissa: 1.0625 is halfway between 1.0 (even) and 1.125
+    assert oq.e4m3_round(np.float32([1.0625, 1.1875, 2.0 ** -10, 3 * 2.0 ** -10])).tolist() == [1.0, 1.25, 0.0, 2 ** -8]
+    # saturation (torch's cast gives NaN above the range; the oracle and the kernels clamp)
+    assert oq.e4m3_round(np.float32([460, 480, 1e6, -1e6])).tolist() == [448.0, 448.0, 448.0, -448.0]
+
+
+def test_block_quant_scales_and_error_bound():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 300, 128, generator=g).to(torch.bfloat16)
+    x[1, 128:256] = 0                                   # an all-zero block
+    codes, scale = oq.dynamic_block_quant(x, 128, 128)
+    assert codes.shape == x.shape and scale.shape == (3, 3, 1) and scale.dtype == torch.float32
+    amax = torch.stack([x[:, i * 128:(i + 1) * 128].float().abs().amax(dim=(1, 2)) for i in range(3)], 1)
+    assert torch.equal(scale[..., 0][amax > 0], (amax / 448.0)[amax > 0]) and scale[1, 1, 0] == 1.0
+    deq = oq.dequant_block(codes, scale, 128, 128)
+    # E4M3 keeps 4 significant bits: relative error <= 2^-4 for normals, absolute <= scale * 2^-10 below
+    err = (deq - x.float()).abs()
+    bound = torch.maximum(x.float().abs() * 2.0 ** -4, scale.repeat_interleave(128, 1)[:, :300] * 2.0 ** -10)
+    assert (err <= bound + 1e-12).all()
+    assert (oq.e4m3_decode(codes.numpy()).__abs__().max() == 448.0)   # the block maximum maps to the largest code
+    c256, s256 = oq.dynamic_block_quant(x, 256, 128)
+    assert s256.shape == (3, 2, 1)
+
+
+def test_per_channel_quant():
+    g = torch.Generator().manual_seed(2)
+    v = torch.randn(2, 500, 128, generator=g) * torch.linspace(0.1, 5, 128)
+    codes, sc = oq.per_channel_quant(v)
+    assert sc.shape == (2, 128) and torch.allclose(sc, v.abs().amax(dim=1) / 448.0)
+    deq = torch.from_numpy(oq.e4m3_decode(codes.numpy())) * sc[:, None, :]
+    assert ((deq - v).abs() <= v.abs() * 2.0 ** -4 + sc[:, None, :] * 2.0 ** -10).all()
+
+
+def test_mx_quant_follows_ocp_mx():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 256, generator=g) * torch.logspace(-3, 3, 64)[:, None]
+    x[5, 32:64] = 0
+    codes, e8 = oq.mx_quant(x)
+    assert codes.shape == (64, 256) and e8.shape == (64, 8) and e8.dtype == torch.uint8
+    amax = x.reshape(64, 8, 32).abs().amax(-1)
+    expect = torch.floor(torch.log2(amax.double().clamp(min=1e-300))) - 8 + 127
+    assert torch.equal(e8.double()[amax > 0], expect[amax > 0]) and e8[5, 1] == 0
+    # the scaled block maximum lies in [256, 512): the top of the E4M3 range, saturated at 448
+    q = torch.from_numpy(oq.e4m3_decode(codes.numpy())).reshape(64, 8, 32).abs().amax(-1)
+    assert ((q >= 256) & (q <= 448))[amax > 0].all()
+    deq = oq.mx_dequant(codes, e8)
+    rel = ((deq - x.double()).abs() / amax.repeat_interleave(32, 1).clamp(min=1e-30)).max()
+    assert rel <= 0.125 + 1e-9        # saturation of [448, 512) costs at most 12.5 % of the block maximum
+    # torch's float8_e8m0fnu agrees on what the scale bytes mean
+    assert torch.equal(e8.view(torch.float8_e8m0fnu).float()[amax > 0],
+                       torch.exp2(e8.float() - 127)[amax > 0])
+
+
+def test_mxfp8_gemm_swiglu_close_to_unquantised():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(96, 512, generator=g)
+    w = torch.randn(2 * 80, 512, generator=g) * 0.02
+    got = oq.mxfp8_gemm_swiglu(x, w, torch.float32)
+    y = x.double() @ w.double().t()
+    want = torch.nn.functional.silu(y[:, :80]) * y[:, 80:]
+    cos = float((got.double().flatten() @ want.flatten()) / (got.double().norm() * want.norm()))
+    assert got.shape == (96, 80) and cos > 0.995
+    # linearity in the power-of-two scale: scaling x by 4 scales the GEMM by exactly 4
+    assert torch.equal(oq.mxfp8_gemm(x * 4, w), oq.mxfp8_gemm(x, w) * 4)
+
+
+def test_fp8_attention_close_to_unquantised():
+    from oracle.attention import attention_fp64, cosine
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 2, 300, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    out = oq.fp8_attention(q, k, v)
+    assert out.dtype == torch.bfloat16
+    for n in range(2):
+        assert cosine(out[0, n], attention_fp64(q[0, n], k[0, n], v[0, n], 128 ** -0.5)) > 0.995
