@@ -1,0 +1,147 @@
+/*
+ * C ABI of libmindiesd_hip.so: the MI355X (gfx950) kernels behind the attention hot path of MindIE-SD.
+ *
+ * Every entry point takes plain device pointers, sizes, element strides and a HIP stream; nothing is
+ * allocated inside (scratch memory, where needed, is an explicit workspace argument with a
+ * *_workspace_size companion, mirroring the aclnnXxxGetWorkspaceSize / aclnnXxx pairs the reference
+ * resolves with dlsym, csrc/plugin/pytorch_npu_helper.h:612-659).  Kernels are enqueued
+ * asynchronously on `stream`; there is no implicit synchronisation.  Inputs are never modified.
+ *
+ * Return value: 0 on success, otherwise
+ *   1  bad argument (null / misaligned pointer, non-positive size, unknown dtype code)
+ *   2  unsupported shape or option (head_dim != 128, offsets beyond 32 bits, ...)
+ *   3  workspace too small
+ *   4  HIP launch failure
+ * (the reference checks the aclnn status the same way: TORCH_CHECK(apiRet == 0, ...),
+ * pytorch_npu_helper.h:646-649).
+ *
+ * dtype codes: 0 = bf16, 1 = fp16.  All tensors have head_dim 128 contiguous in memory; pointers must
+ * be 16-byte aligned and every stride a multiple of 8 elements.  "strides" are element strides of the
+ * (batch, head, token) dimensions, so BNSD and BSND tensors are both passed without a copy.
+ */
+#ifndef MINDIESD_HIP_H
+#define MINDIESD_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* hipStream_t;
+
+/* ---- dense attention -------------------------------------------------------------------------------
+ * out = softmax(scale * Q K^T) V per (batch, head); N % Nkv == 0 (grouped-query heads).
+ * lse: optional [B][N][Sq] fp32 log-sum-exp of the scaled scores (may be NULL).
+ * Replaces the fused kernels behind attention_forward
+ * (mindiesd/layers/flash_attn/attention_forward.py:24-89: torch_npu.npu_prompt_flash_attention
+ * prompt_flash_attn.py:48, npu_fusion_attention fused_attn_score.py:48, torch.ops.mindiesd.la
+ * csrc/plugin/la.cpp:27-58). */
+int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                 int B, int N, int Nkv, int Sq, int Skv, int D,
+                                 long long q_sb, long long q_sn, long long q_ss,
+                                 long long k_sb, long long k_sn, long long k_ss,
+                                 long long v_sb, long long v_sn, long long v_ss,
+                                 long long o_sb, long long o_sn, long long o_ss,
+                                 float scale, hipStream_t stream);
+
+/* Benchmark hook: selects one of the compiled dense kernel variants (0 = default). */
+void mindiesd_set_dense_variant(int variant);
+
+/* ---- block-sparse attention ------------------------------------------------------------------------
+ * Query block i (128 rows) of (b, n) attends to the 128-key blocks blk_idx[b][n][i][0 .. blk_cnt[b][n][i])
+ * (ascending ids, int32, row pitch kb_stride); an empty list gives zeros.  `order` (optional,
+ * [B*N*ceil(Sq/128)]) is the sequence in which query blocks are dispatched.
+ * Replaces aclnnBlockSparseAttention / aclnnRainFusionAttention behind
+ * torch.ops.mindiesd.block_sparse_attention / rainfusionattention
+ * (csrc/plugin/block_sparse_attention.cpp:31-121, csrc/plugin/rainfusionattention.cpp:27-64). */
+int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                        int B, int N, int Nkv, int Sq, int Skv, int D,
+                                        long long q_sb, long long q_sn, long long q_ss,
+                                        long long k_sb, long long k_sn, long long k_ss,
+                                        long long v_sb, long long v_sn, long long v_ss,
+                                        long long o_sb, long long o_sn, long long o_ss,
+                                        float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                        const int* order, hipStream_t stream);
+
+/* ---- RainFusion2.0 mask pipeline ---------------------------------------------------------------------
+ * Token permutation into 8x8 spatial windows (+ optional block mean pooling) of up to three tensors
+ * of one shape; replaces rearrange_with_remaining / avgpool / do_tensor_rearrange_pooling /
+ * inv_rearrange_with_remaining (mindiesd/layers/flash_attn/sparse_flash_attn_rf_v2.py:24-73,
+ * :137-317).  The sequence is [txt_len text tokens | t*h*w image tokens]; the permuted sequence is
+ * [image in window order | text].  t == 0 selects the identity order (pooling only).  inverse != 0
+ * undoes the permutation.  q_out/k_out/v_out may be NULL (pool only); pool may be NULL (permute only).
+ * pool: 16-bit [n_tensors][B][N][blocks][128] addressed with strides p_st (tensor), p_sb, p_sn,
+ * p_sblk; blocks = ceil(image/128) + ceil(text/128), each block averaged over its own length. */
+int mindiesd_rf_rearrange_pool(const void* q, const void* k, const void* v, void* q_out, void* k_out, void* v_out,
+                               void* pool, int dtype, int B, int N, int S, int D,
+                               long long s_sb, long long s_sn, long long s_ss,
+                               long long d_sb, long long d_sn, long long d_ss,
+                               long long p_st, long long p_sb, long long p_sn, long long p_sblk,
+                               int t, int h, int w, int txt_len, int inverse, int n_tensors, hipStream_t stream);
+
+/* Block mask from pooled q/k (get_blockwise_mask + get_mask_index, sparse_flash_attn_rf_v2.py:76-134):
+ * keep[b][n][i][j] = softmax_j(q_pool_i . k_pool_j * scale) >= keep_len-th largest of row i,
+ * OR i/j inside the last txt_blocks or the first ff_blocks blocks, OR (keep_diag and i == j);
+ * scores and probabilities are rounded to the 16-bit input type at the reference's rounding points.
+ * Outputs (each optional): mask int8 [B][N][NB][NB]; blk_idx int32 [B][N][NB][kb_stride] ascending,
+ * -1 padded, with blk_cnt int32 [B][N][NB]; select_idx int64 [NB][N][NB] / select_num int64 [NB][N]
+ * (batch 0, the reference's layout). */
+int mindiesd_rf_block_mask(const void* q_pool, const void* k_pool, int dtype, int B, int N, int NB, int D,
+                           long long p_sb, long long p_sn, long long p_sblk, float scale, int keep_len,
+                           int txt_blocks, int ff_blocks, int keep_diag, signed char* mask, int* blk_idx,
+                           int* blk_cnt, int kb_stride, long long* select_idx, long long* select_num,
+                           hipStream_t stream);
+
+/* int8 mask [BN][QB][KB] (non-zero = attend) -> ascending index lists + counts (the form
+ * mindiesd_block_sparse_attention_fwd consumes). */
+int mindiesd_mask_to_index(const signed char* mask, int BN, int QB, int KB, int* blk_idx, int* blk_cnt,
+                           int kb_stride, hipStream_t stream);
+
+/* Dispatch order for the block-sparse kernel: query blocks sorted by descending block count. */
+int mindiesd_lpt_order(const int* blk_cnt, int* order, int total, int max_cnt, hipStream_t stream);
+
+/* ---- FP8 attention -----------------------------------------------------------------------------------
+ * Block quantisation of one attention operand: x [B][N][S][128] 16-bit (strided) ->
+ * q [B][N][S][128] E4M3 bytes + scale fp32 [B][N][ceil(S/block_size)], scale = amax/448 per block of
+ * block_size (128/256/512) tokens x 128 channels.  Replaces torch_npu.npu_dynamic_block_quant as
+ * called by fa_block_quant_preprocess (mindiesd/layers/quant/block_quant.py:19-48). */
+int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int B, int N, int S, int D,
+                            long long x_sb, long long x_sn, long long x_ss, int block_size, hipStream_t stream);
+
+/* V for the FP8 kernel: per-(batch, head, channel) scale = amax/448 over the sequence, codes written
+ * transposed ([B][N][128][S rounded up to 128], zero padded, keys permuted inside groups of 64 into
+ * the order the matrix instruction consumes).  workspace: mindiesd_fp8_v_quant_workspace_size bytes. */
+size_t mindiesd_fp8_v_quant_workspace_size(int B, int N);
+int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
+                         long long v_sb, long long v_sn, long long v_ss, void* workspace, size_t ws_bytes,
+                         hipStream_t stream);
+
+/* FP8 flash attention on operands produced by the two functions above (Q/K with block_size 128).
+ * Replaces torch_npu.npu_fused_infer_attention_score_v2 with per-block dequantisation scales as
+ * called by FP8RotateQuantFA.forward (mindiesd/quantization/layer.py:304-316). */
+int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
+                               const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
+                               int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,
+                               hipStream_t stream);
+
+/* ---- MXFP8 linear layer --------------------------------------------------------------------------------
+ * x [M][K] 16-bit (row stride x_stride elements) -> q [M][K] E4M3 + e8m0 [M][K/32]
+ * (OCP MX: shared scale 2^(floor(log2(amax)) - 8) per 32 elements).  Replaces
+ * torch_npu.npu_dynamic_mx_quant (mindiesd/quantization/layer.py:338-341). */
+int mindiesd_mx_quant(const void* x, void* q, void* e8m0, int dtype, long long M, int K, long long x_stride,
+                      hipStream_t stream);
+
+/* out[M][Nout] = act(X W^T + bias) on MX-quantised operands (a [M][K], a_scale [M][K/32], w [Nw][K],
+ * w_scale [Nw][K/32], bias fp32 [Nw] or NULL).  swiglu == 0: Nout = Nw.  swiglu != 0: W holds
+ * [gate rows | up rows], Nout = Nw/2 and out = silu(gate) * up, computed on the accumulators.
+ * Replaces torch_npu.npu_quant_matmul(..., group_sizes=[1,1,32]) (mindiesd/quantization/layer.py:351-361);
+ * the fused SwiGLU has no counterpart in the reference, which applies nn.SiLU afterwards
+ * (mindiesd/layers/activation.py:34-61). */
+int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const void* w_scale, const float* bias,
+                        void* out, int out_dtype, int M, int K, int Nw, int swiglu, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINDIESD_HIP_H */

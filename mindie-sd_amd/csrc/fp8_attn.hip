@@ -1,0 +1,501 @@
+// FP8 (OCP E4M3) attention for gfx950 (MI355X): quantisation passes + flash-attention forward on
+// the fp8 matrix cores (v_mfma_f32_32x32x64_f8f6f4, twice the bf16 rate).
+//
+// Takes the place of the vendor ops behind the reference's FP8 attention path:
+//   fa_block_quant_preprocess / npu_dynamic_block_quant   mindiesd/layers/quant/block_quant.py:19-48
+//   FP8RotateQuantFA -> npu_fused_infer_attention_score_v2 mindiesd/quantization/layer.py:283-324
+//
+// Recipe (Wan2.1-14B 480p workload): Q and K as E4M3 with one fp32 scale per (head, 128-token block)
+// over all 128 channels, V as E4M3 with one fp32 scale per (head, channel), P re-quantised to E4M3
+// per tile, fp32 accumulation, 16-bit output.
+//
+// Layouts produced by the quantisation pass and consumed by the attention kernel:
+//   Q8, K8 : [B][N][S][128] bytes, row major.
+//   V8T    : [B][N][128][S128] bytes (S rounded up to 128, zero padded), i.e. V transposed so that
+//            a lane of the second product reads its 32 keys as 32 contiguous bytes.  Inside every
+//            group of 64 keys the keys are stored in the order in which the S^T accumulator of the
+//            first product hands them to the second one: position 32*h + j holds key
+//            32*(j/16) + 8*((j%16)/4) + 4*h + j%4   (h = 0,1 the wave half, j = 0..31).
+#include "common.hpp"
+
+namespace msd {
+
+constexpr float kE4M3Max = 448.0f;
+
+__device__ __forceinline__ float clamp448(float x) { return __builtin_amdgcn_fmed3f(x, -kE4M3Max, kE4M3Max); }
+
+// four floats -> four E4M3 bytes (RNE, saturating), first value in the lowest byte
+__device__ __forceinline__ int pack4_e4m3(float a, float b, float c, float d) {
+  int w = 0;
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(a), clamp448(b), w, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(c), clamp448(d), w, true);
+  return w;
+}
+// probabilities are already inside the range: no clamp
+__device__ __forceinline__ int pack4_e4m3_noclamp(float a, float b, float c, float d) {
+  int w = 0;
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return w;
+}
+
+template <int DT>
+__device__ __forceinline__ void load8(const typename Elem<DT>::type* p, float (&f)[8]) {
+  union { i32x4_t v; typename Elem<DT>::type e[8]; } u;
+  u.v = *(const i32x4_t*)p;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) f[j] = (float)u.e[j];
+}
+
+__device__ __forceinline__ float block_max_256(float v, float* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return v;
+}
+
+// ---- block quantisation: one scale per (batch, head, `bs` tokens) over all 128 channels --------------
+// x [B][N][S][128] (strided) -> q [B][N][S][128] bytes (contiguous), scale [B][N][ceil(S/bs)].
+template <int DT>
+__global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsigned char* q, float* scale,
+                                                          long long sb, long long sn, long long ss, int N, int S,
+                                                          int bs) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using T = typename Elem<DT>::type;
+  __shared__ float red[4];
+  const int blk = blockIdx.x, bn = blockIdx.y;
+  const int b = bn / N, n = bn - b * N;
+  const int nblk = gridDim.x;
+  const T* x = (const T*)x_ + b * sb + n * sn;
+  const int row0 = blk * bs, rows = min(bs, S - row0);
+  const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
+  float amax = 0.f;
+  for (int r = rgrp; r < rows; r += 16) {
+    float f[8];
+    load8<DT>(x + (long long)(row0 + r) * ss + c16 * 8, f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
+  }
+  amax = block_max_256(amax, red);
+  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  if (threadIdx.x == 0) scale[(long long)bn * nblk + blk] = sc;
+  unsigned char* qo = q + ((long long)bn * S + row0) * 128 + c16 * 8;
+  for (int r = rgrp; r < rows; r += 16) {
+    float f[8];
+    load8<DT>(x + (long long)(row0 + r) * ss + c16 * 8, f);   // second read hits L2
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn(f[j], sc);
+    i32x2_t w = {pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
+    *(i32x2_t*)(qo + (long long)r * 128) = w;
+  }
+#endif
+}
+
+// ---- V: per-channel maximum over the sequence ------------------------------------------------------------
+__global__ void fill_u32_kernel(unsigned* p, unsigned v, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// amax_bits [B][N][128] must be zero-filled; non-negative floats order like their bit patterns.
+template <int DT>
+__global__ __launch_bounds__(256) void channel_amax_kernel(const void* v_, unsigned* amax_bits, long long sb,
+                                                           long long sn, long long ss, int N, int S) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using T = typename Elem<DT>::type;
+  __shared__ float part[16][128];
+  const int bn = blockIdx.y, b = bn / N, n = bn - b * N;
+  const T* v = (const T*)v_ + b * sb + n * sn;
+  const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
+  const int row0 = blockIdx.x * 1024, rows = min(1024, S - row0);
+  float m[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) m[j] = 0.f;
+  for (int r = rgrp; r < rows; r += 16) {
+    float f[8];
+    load8<DT>(v + (long long)(row0 + r) * ss + c16 * 8, f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m[j] = fmaxf(m[j], fabsf(f[j]));
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) part[rgrp][c16 * 8 + j] = m[j];
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    float a = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) a = fmaxf(a, part[r][threadIdx.x]);
+    atomicMax(amax_bits + (long long)bn * 128 + threadIdx.x, __builtin_bit_cast(unsigned, a));
+  }
+#endif
+}
+
+// position of key kk (0..63) inside its 64-key group of V8T
+__host__ __device__ __forceinline__ int v8t_pos(int kk) {
+  const int blk32 = kk >> 5, r = kk & 31;
+  const int g8 = r >> 3, within = r & 7;
+  const int h = within >> 2, e = within & 3;
+  return 32 * h + 16 * blk32 + 4 * g8 + e;
+}
+
+// V [B][N][S][128] -> V8T [B][N][128][S128] bytes + per-channel scale [B][N][128] = amax/448.
+// One workgroup = 64 keys of one (batch, head).
+template <int DT>
+__global__ __launch_bounds__(256) void v_quant_transpose_kernel(const void* v_, const unsigned* amax_bits,
+                                                                unsigned char* v8t, float* vscale, long long sb,
+                                                                long long sn, long long ss, int N, int S, int S128) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using T = typename Elem<DT>::type;
+  __shared__ unsigned char tile[128][64 + 16];  // [channel][position], padded rows
+  const int grp = blockIdx.x, bn = blockIdx.y, b = bn / N, n = bn - b * N;
+  const T* v = (const T*)v_ + b * sb + n * sn;
+  const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
+  float sc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a = __builtin_bit_cast(float, amax_bits[(long long)bn * 128 + c16 * 8 + j]);
+    sc[j] = a > 0.f ? __fdiv_rn(a, kE4M3Max) : 1.0f;
+  }
+  if (grp == 0 && rgrp == 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vscale[(long long)bn * 128 + c16 * 8 + j] = sc[j];
+  }
+  for (int kk = rgrp; kk < 64; kk += 16) {
+    const int key = grp * 64 + kk;
+    float f[8];
+    if (key < S) {
+      load8<DT>(v + (long long)key * ss + c16 * 8, f);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = 0.f;
+    }
+    const int pos = v8t_pos(kk);
+#pragma unroll
+    for (int j = 0; j < 8; j += 4) {
+      const int w = pack4_e4m3(__fdiv_rn(f[j], sc[j]), __fdiv_rn(f[j + 1], sc[j + 1]), __fdiv_rn(f[j + 2], sc[j + 2]),
+                               __fdiv_rn(f[j + 3], sc[j + 3]));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) tile[c16 * 8 + j + e][pos] = (unsigned char)((unsigned)w >> (8 * e));
+    }
+  }
+  __syncthreads();
+  // 128 channel rows x 64 bytes: 4 lanes write one row
+  for (int i = threadIdx.x; i < 128 * 4; i += 256) {
+    const int ch = i >> 2, part = i & 3;
+    const i32x4_t w = *(const i32x4_t*)&tile[ch][part * 16];
+    *(i32x4_t*)(v8t + ((long long)bn * 128 + ch) * S128 + grp * 64 + part * 16) = w;
+  }
+#endif
+}
+
+// ---- attention ------------------------------------------------------------------------------------------------
+struct Fp8Params {
+  const unsigned char* q8;
+  const unsigned char* k8;
+  const unsigned char* v8t;
+  const float* q_scale;  // [B][N][ceil(Sq/128)]
+  const float* k_scale;  // [B][N][ceil(Skv/128)]
+  const float* v_scale;  // [B][N][128]
+  void* o;
+  long long o_sb, o_sn, o_ss;
+  int B, N, Sq, Skv, S128;
+  float scale_log2;  // softmax scale * log2(e)
+};
+
+// P is scaled by 2^kPShift before the E4M3 conversion; with the lazy-maximum threshold kTau8 the
+// largest value is 2^(kTau8 + kPShift) = 256 <= 448 and values down to 2^-13 survive as subnormals.
+constexpr float kTau8 = 4.0f;
+constexpr float kPShift = 4.0f;
+
+// 8 waves x 32 query rows, 128-key tiles, K tile [key][128 B] and V^T tile [channel][128 B] in LDS
+// (16 KiB each, double buffered); 16-byte chunk c of row r is stored at chunk c ^ ((r >> 1) & 7).
+template <int DT>
+__global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using E = Elem<DT>;
+  using T = typename E::type;
+  constexpr int NW = 8, BM = 256, BN = 128;
+  constexpr int kTile = BN * 128;        // bytes of one K (or V^T) tile
+  constexpr int kStage = 2 * kTile;
+  constexpr int kORow = 256 + 8;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  MSD_LDS char* smem = (MSD_LDS char*)smem_raw;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, h = lane >> 5;
+
+  const int q_tiles = (p.Sq + BM - 1) / BM;
+  const int total = p.B * p.N * q_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (work >= total) return;
+  const int bn = work / q_tiles, qt = work - bn * q_tiles;
+  const int b = bn / p.N, n = bn - b * p.N;
+  const int q0 = qt * BM;
+  const int qblocks = (p.Sq + 127) / 128, kblocks = (p.Skv + 127) / 128;
+  const int n_tiles = kblocks;
+
+  // Q^T operand: lane (q = l32, h) holds bytes 64*ks + 32*h .. +32 of its row
+  const int qrow = q0 + wave * 32 + l32;
+  const bool q_ok = qrow < p.Sq;
+  const unsigned char* qsrc = p.q8 + ((long long)bn * p.Sq + (q_ok ? qrow : 0)) * 128 + 32 * h;
+  i32x8_t qf[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    const i32x4_t lo = *(const i32x4_t*)(qsrc + 64 * ks), hi = *(const i32x4_t*)(qsrc + 64 * ks + 16);
+    qf[ks] = q_ok ? i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]} : i32x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  // all 32 rows of a wave lie in one 128-row scale block
+  const int qblk = min((q0 + wave * 32) >> 7, qblocks - 1);
+  const float q_sc = p.q_scale[(long long)bn * qblocks + qblk] * p.scale_log2;
+  const float* k_sc = p.k_scale + (long long)bn * kblocks;
+
+  f32x16_t oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // ---- LDS-DMA staging: one instruction = 8 rows x 128 bytes ----------------------------------------------------
+  const unsigned char* kg = p.k8 + (long long)bn * p.Skv * 128;
+  const unsigned char* vg = p.v8t + (long long)bn * 128 * p.S128;
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, p.Skv * 128, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, 128 * p.S128, 0x00020000);
+  int k_voff[2], v_voff[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = 8 * (i * NW + wave) + (lane >> 3);
+    const int c = (lane & 7) ^ ((row >> 1) & 7);
+    k_voff[i] = row * 128 + c * 16;          // + key0 * 128 (scalar)
+    v_voff[i] = row * p.S128 + c * 16;       // + key0 (scalar); row = channel
+  }
+  auto load_tile = [&](int t, int stage) {
+    MSD_LDS char* kb = smem + stage * kStage;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int g = i * NW + wave;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g * 1024), 16, k_voff[i], t * BN * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(kb + kTile + g * 1024), 16, v_voff[i], t * BN, 0,
+                                               0);
+    }
+  };
+
+  // operand read offsets: row = blk*32 + l32, bytes 64*ks + 32*h .. +32 = chunks 4*ks + 2*h, +1
+  const int row_off = l32 * 128;
+  const int swz = (l32 >> 1) & 7;
+
+  if (n_tiles > 0) load_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+
+  for (int t = 0; t < n_tiles; ++t) {
+    const int stage = t & 1;
+    if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
+    MSD_LDS const char* kb_base = smem + stage * kStage;
+    MSD_LDS const char* vb_base = kb_base + kTile;
+
+    // ---- S^T = K Q^T (fp8, unscaled form of the scaled MFMA) ---------------------------------------------------
+    f32x16_t sacc[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        MSD_LDS const char* src = kb_base + kb * 32 * 128 + row_off;
+        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h) ^ swz) << 4));
+        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h + 1) ^ swz) << 4));
+        const i32x8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
+      }
+    }
+
+    const int key0 = t * BN;
+    if (key0 + BN > p.Skv) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3) >= p.Skv) sacc[kb][r] = -INFINITY;
+    }
+
+    // ---- online softmax (exp2 domain, lazily updated reference maximum), P -> E4M3 ------------------------------
+    const float c = q_sc * k_sc[t];  // dequantisation scales of this tile folded into the softmax scale
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+    mx = half_max(mx) * c;
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau8) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
+    const float mc = (m_run == -INFINITY ? 0.f : m_run) - kPShift;
+    float ls = 0.f;
+    i32x8_t pf[2];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = fast_exp2(__builtin_fmaf(sacc[kb][r], c, -mc));
+        ls += e;
+        sacc[kb][r] = e;
+      }
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4)
+        pf[kb >> 1][(kb & 1) * 4 + g4] =
+            pack4_e4m3_noclamp(sacc[kb][4 * g4], sacc[kb][4 * g4 + 1], sacc[kb][4 * g4 + 2], sacc[kb][4 * g4 + 3]);
+    }
+    l_run += ls;
+
+    // ---- O^T += V^T P^T (fp8) ---------------------------------------------------------------------------------------
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        MSD_LDS const char* src = vb_base + db * 32 * 128 + row_off;
+        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(src + (((4 * kk + 2 * h) ^ swz) << 4));
+        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(src + (((4 * kk + 2 * h + 1) ^ swz) << 4));
+        const i32x8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf[kk], oacc[db], 0, 0, 0, 0, 0, 0);
+      }
+    }
+
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+  }
+
+  // ---- epilogue: 1/l, per-channel V scale, transpose through LDS, coalesced store -----------------------------------
+  // (the 2^kPShift factor is in both the accumulator and the running sum, so it cancels)
+  const float l_tot = half_sum(l_run);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const float* vs = p.v_scale + (long long)bn * 128;
+  MSD_LDS char* ost = smem + wave * 32 * kORow;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = db * 32 + 8 * g + 4 * h;
+      const f32x4_t sv = *(const f32x4_t*)(vs + d);
+      typename E::x4 pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[j] = E::from_float(oacc[db][4 * g + j] * inv * sv[j]);
+      *(MSD_LDS typename E::x4*)(ost + l32 * kORow + d * 2) = pk;
+    }
+  __builtin_amdgcn_wave_barrier();
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int cidx = i * 64 + lane;
+    const int row = cidx >> 4, c16 = cidx & 15;
+    const int qr = q0 + wave * 32 + row;
+    const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16);
+    const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16 + 8);
+    if (qr < p.Sq) *(i32x4_t*)(og + (long long)qr * p.o_ss + c16 * 8) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
+  }
+#endif
+}
+
+}  // namespace msd
+
+using namespace msd;
+
+extern "C" {
+
+int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int B, int N, int S, int D,
+                            long long x_sb, long long x_sn, long long x_ss, int block_size, hipStream_t stream) {
+  if (!x || !q || !scale || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (block_size != 128 && block_size != 256 && block_size != 512) return MSD_ERR_BAD_ARG;
+  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if (((uintptr_t)x & 15) || ((uintptr_t)q & 7) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
+  dim3 grid((S + block_size - 1) / block_size, B * N);
+  if (dtype == MSD_DTYPE_BF16)
+    hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
+                       x_sn, x_ss, N, S, block_size);
+  else
+    hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
+                       x_sn, x_ss, N, S, block_size);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+// bytes of the caller-provided scratch for mindiesd_fp8_v_quant (per-channel maxima)
+size_t mindiesd_fp8_v_quant_workspace_size(int B, int N) { return (size_t)B * N * 128 * sizeof(unsigned); }
+
+int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
+                         long long v_sb, long long v_sn, long long v_ss, void* workspace, size_t ws_bytes,
+                         hipStream_t stream) {
+  if (!v || !v8t || !v_scale || !workspace || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if (ws_bytes < mindiesd_fp8_v_quant_workspace_size(B, N)) return MSD_ERR_WORKSPACE;
+  if (((uintptr_t)v & 15) || ((uintptr_t)v8t & 15) || ((v_sb | v_sn | v_ss) & 7)) return MSD_ERR_BAD_ARG;
+  const long long nbits = (long long)B * N * 128;
+  const int S128 = (S + 127) / 128 * 128;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nbits + 255) / 256)), dim3(256), 0, stream, (unsigned*)workspace,
+                     0u, nbits);
+  dim3 g1((S + 1023) / 1024, B * N), g2(S128 / 64, B * N);
+  if (dtype == MSD_DTYPE_BF16) {
+    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_BF16>, g1, dim3(256), 0, stream, v, (unsigned*)workspace, v_sb, v_sn,
+                       v_ss, N, S);
+    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_BF16>, g2, dim3(256), 0, stream, v,
+                       (const unsigned*)workspace, (unsigned char*)v8t, v_scale, v_sb, v_sn, v_ss, N, S, S128);
+  } else {
+    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_F16>, g1, dim3(256), 0, stream, v, (unsigned*)workspace, v_sb, v_sn,
+                       v_ss, N, S);
+    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_F16>, g2, dim3(256), 0, stream, v, (const unsigned*)workspace,
+                       (unsigned char*)v8t, v_scale, v_sb, v_sn, v_ss, N, S, S128);
+  }
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
+                               const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
+                               int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,
+                               hipStream_t stream) {
+  if (!q8 || !k8 || !v8t || !q_scale || !k_scale || !v_scale || !out) return MSD_ERR_BAD_ARG;
+  if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return MSD_ERR_BAD_ARG;
+  if (D != 128 || !(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
+  if (out_dtype != MSD_DTYPE_BF16 && out_dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if (((uintptr_t)q8 | (uintptr_t)k8 | (uintptr_t)v8t | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
+  if ((o_sb | o_sn | o_ss) & 7) return MSD_ERR_BAD_ARG;
+  const int S128 = (Skv + 127) / 128 * 128;
+  if ((long long)Skv * 128 >= (1ll << 31) || 128ll * S128 >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
+  Fp8Params p{};
+  p.q8 = (const unsigned char*)q8; p.k8 = (const unsigned char*)k8; p.v8t = (const unsigned char*)v8t;
+  p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale;
+  p.o = out; p.o_sb = o_sb; p.o_sn = o_sn; p.o_ss = o_ss;
+  p.B = B; p.N = N; p.Sq = Sq; p.Skv = Skv; p.S128 = S128;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  constexpr int kLds = 8 * 32 * (256 + 8);  // output staging (66 KiB) > 2 stages x 32 KiB
+  const int q_tiles = (Sq + 255) / 256;
+  const int total = B * N * q_tiles;
+  const int grid = (total + 7) / 8 * 8;
+  if (out_dtype == MSD_DTYPE_BF16) {
+    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16>;
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+      return MSD_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
+  } else {
+    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16>;
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+      return MSD_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
+  }
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+}  // extern "C"

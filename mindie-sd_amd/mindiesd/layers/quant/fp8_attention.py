@@ -1,0 +1,70 @@
+"""FP8 attention on the MI355X fp8 matrix cores.
+
+Stands where the reference calls ``torch_npu.npu_fused_infer_attention_score_v2`` with per-block
+dequantisation scales (mindiesd/quantization/layer.py:297-316).  Recipe: Q and K E4M3 with one fp32
+scale per (head, 128-token block), V E4M3 with one scale per (head, channel), probabilities
+re-quantised to E4M3 per tile, fp32 accumulation, output in the input dtype."""
+import torch
+
+from ... import _native
+from ...utils.exception import ParametersInvalid
+from ..flash_attn.hip_flash_attn import HEAD_DIM, _strides_bns
+from .block_quant import _block_quant
+
+
+def quantize_v_per_channel(value, layout="BNSD"):
+    """value [B,N,S,128] / [B,S,N,128] -> (V8T uint8 [B, N, 128, S128] in the kernel's transposed,
+    key-permuted layout, fp32 per-channel scale [B, N, 128])."""
+    if value.dtype not in _native.DTYPE_CODE or not value.is_cuda:
+        raise ParametersInvalid(f"fp8 attention needs bf16/fp16 GPU tensors, but got {value.dtype} on {value.device}.")
+    ok = value.stride(-1) == 1 and value.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in value.stride()[:-1])
+    v = value if ok else value.contiguous()
+    b, n, s = (v.shape[0], v.shape[1], v.shape[2]) if layout == "BNSD" else (v.shape[0], v.shape[2], v.shape[1])
+    s128 = (s + 127) // 128 * 128
+    v8t = torch.empty((b, n, HEAD_DIM, s128), dtype=torch.uint8, device=v.device)
+    vscale = torch.empty((b, n, HEAD_DIM), dtype=torch.float32, device=v.device)
+    lib = _native.lib()
+    ws = torch.empty(lib.mindiesd_fp8_v_quant_workspace_size(b, n), dtype=torch.uint8, device=v.device)
+    with torch.cuda.device(v.device):
+        rc = lib.mindiesd_fp8_v_quant(v.data_ptr(), v8t.data_ptr(), vscale.data_ptr(), _native.DTYPE_CODE[v.dtype],
+                                      b, n, s, HEAD_DIM, *_strides_bns(v, layout), ws.data_ptr(), ws.numel(),
+                                      _native.stream_ptr(v.device))
+    _native.check(rc, "mindiesd_fp8_v_quant")
+    return v8t, vscale
+
+
+def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_dtype=torch.bfloat16, layout="BNSD"):
+    """Attention on already quantised operands (see ``quantize_v_per_channel`` and ``_block_quant``
+    with block 128).  Output [B,N,S,128] ('BNSD') or [B,S,N,128] ('BSND') in ``out_dtype``."""
+    b, n, sq, d = q8.shape
+    skv = k8.shape[2]
+    shape = (b, n, sq, d) if layout == "BNSD" else (b, sq, n, d)
+    out = torch.empty(shape, dtype=out_dtype, device=q8.device)
+    with torch.cuda.device(q8.device):
+        rc = _native.lib().mindiesd_fp8_attention_fwd(
+            q8.data_ptr(), k8.data_ptr(), v8t.data_ptr(), q_scale.data_ptr(), k_scale.data_ptr(), v_scale.data_ptr(),
+            out.data_ptr(), _native.DTYPE_CODE[out_dtype], b, n, sq, skv, d, *_strides_bns(out, layout),
+            float(scale), _native.stream_ptr(q8.device))
+    _native.check(rc, "mindiesd_fp8_attention_fwd")
+    return out
+
+
+def fp8_attention_forward(query, key, value, scale=None, layout="BNSD"):
+    """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``."""
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        if not isinstance(t, torch.Tensor) or t.dim() != 4:
+            raise ParametersInvalid(f"The input {name} must be a 4-D torch.Tensor.")
+    if layout not in ("BNSD", "BSND"):
+        raise ParametersInvalid(f"Unsupported layout: {layout}, expected 'BNSD' or 'BSND'.")
+    if key.shape != value.shape or query.shape[-1] != HEAD_DIM or key.shape[-1] != HEAD_DIM:
+        raise ParametersInvalid("fp8 attention needs head_dim 128 and equal key/value shapes.")
+    nq = query.shape[1] if layout == "BNSD" else query.shape[2]
+    nk = key.shape[1] if layout == "BNSD" else key.shape[2]
+    if nq != nk or query.shape[0] != key.shape[0]:
+        raise ParametersInvalid("fp8 attention needs the same batch and head count for query and key/value.")
+    if scale is None:
+        scale = query.shape[-1] ** -0.5
+    q8, qs = _block_quant(query, 128, layout)
+    k8, ks = _block_quant(key, 128, layout)
+    v8t, vs = quantize_v_per_channel(value, layout)
+    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout)

@@ -1,0 +1,107 @@
+"""GPU parity of the FP8 path vs the CPU oracle: quantised codes and scales bit-exact against the
+format definition (OCP E4M3, scale = amax/448), attention output cosine >= 0.999 against the
+quantise -> dequantise oracle (the stated tolerance of the FP8 workload)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from oracle.attention import cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def _outlier_inputs(shape, seed, dtype=torch.bfloat16):
+    """N(0,1) with 1 % of the elements scaled by 8 (the FP8 workload's input recipe)."""
+    g = torch.Generator().manual_seed(seed)
+    outs = []
+    for _ in range(3):
+        x = torch.randn(shape, generator=g)
+        x = torch.where(torch.rand(shape, generator=g) < 0.01, x * 8, x)
+        outs.append(x.to(dtype))
+    return outs
+
+
+@pytest.mark.parametrize("layout", ["BNSD", "BSND"])
+@pytest.mark.parametrize("block", [128, 256, 512])
+def test_block_quant_bit_exact(cuda, block, layout):
+    from mindiesd.layers.quant import fa_block_quant_preprocess
+    x = _outlier_inputs((1, 3, 1000, 128), seed=block)[0]
+    x[0, 1, 256:384] = 0                      # an all-zero block
+    xin = x if layout == "BNSD" else x.transpose(1, 2).contiguous()
+    q, scale = fa_block_quant_preprocess(xin.to(cuda), block_size=block, layout=layout)
+    codes, want_scale = oq.dynamic_block_quant(x, block, 128)
+    assert q.dtype == torch.float8_e4m3fn and q.shape == (1, 3, 1000, 128)
+    assert scale.shape == (1, 3, (1000 + block - 1) // block, 1) and scale.dtype == torch.float32
+    assert torch.equal(scale.cpu(), want_scale)
+    got = q.view(torch.uint8).cpu()
+    same = got == codes
+    # -0 / +0 codes are the same number
+    zero = ((got & 0x7f) == 0) & ((codes & 0x7f) == 0)
+    assert bool((same | zero).all()), f"{(~(same | zero)).sum().item()} codes differ"
+
+
+def test_block_quant_fp16_and_errors(cuda):
+    from mindiesd import ParametersInvalid
+    from mindiesd.layers.quant import fa_block_quant_preprocess
+    x = _outlier_inputs((2, 2, 300, 128), seed=3, dtype=torch.float16)[0]
+    q, scale = fa_block_quant_preprocess(x.to(cuda))
+    codes, want_scale = oq.dynamic_block_quant(x, 128, 128)
+    assert torch.equal(scale.cpu()[..., 0], want_scale[..., 0])
+    assert torch.equal(q.view(torch.uint8).cpu() & 0x7f, codes & 0x7f)
+    with pytest.raises(ParametersInvalid):
+        fa_block_quant_preprocess(x[0].to(cuda))
+    with pytest.raises(ParametersInvalid):
+        fa_block_quant_preprocess(x.to(cuda), block_size=64)
+
+
+def test_v_per_channel_quant_bit_exact(cuda):
+    from mindiesd.layers.quant.fp8_attention import quantize_v_per_channel
+    v = _outlier_inputs((1, 2, 333, 128), seed=5)[2]
+    v8t, vs = quantize_v_per_channel(v.to(cuda))
+    codes, want = oq.per_channel_quant(v)
+    assert torch.equal(vs.cpu(), want)
+    assert v8t.shape == (1, 2, 128, 384)
+    # undo the kernel's layout: position 32*h + j of each 64-key group holds key 32*(j/16) + 8*((j%16)/4) + 4*h + j%4
+    pos = np.empty(64, dtype=np.int64)
+    for h in range(2):
+        for j in range(32):
+            pos[32 * (j // 16) + 8 * ((j % 16) // 4) + 4 * h + j % 4] = 32 * h + j
+    got = v8t.cpu().numpy().reshape(1, 2, 128, 6, 64)[..., pos].reshape(1, 2, 128, 384).transpose(0, 1, 3, 2)
+    assert np.array_equal(got[:, :, :333] & 0x7f, codes.numpy() & 0x7f)
+    assert (got[:, :, 333:] & 0x7f == 0).all(), "padding keys must be zero"
+
+
+@pytest.mark.parametrize("layout,s", [("BNSD", 1024), ("BNSD", 1100), ("BSND", 700)])
+def test_fp8_attention_vs_oracle(cuda, layout, s):
+    from mindiesd.layers.quant import fp8_attention_forward
+    q, k, v = _outlier_inputs((1, 3, s, 128), seed=s)
+    want = oq.fp8_attention(q, k, v)
+    args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout).cpu()
+    out = out if layout == "BNSD" else out.transpose(1, 2)
+    assert out.dtype == torch.bfloat16 and out.shape == q.shape
+    cos = cosine(out, want)
+    err = (out.float() - want.float()).abs()
+    print(f"fp8 attention S={s} {layout}: cosine {cos:.6f}, max-abs {err.max():.4f}, mean-abs {err.mean():.5f}, "
+          f"output rms {want.float().pow(2).mean().sqrt():.4f}")
+    assert cos >= 0.999, f"cosine {cos}"
+    # coarse guard against gross outliers: E4M3 probabilities carry 2^-4 relative noise per element
+    assert err.max() < 0.2 * want.float().abs().max()
+
+
+def test_fp8_rotate_quant_fa_module(cuda):
+    """The reference's module shape (mindiesd/quantization/layer.py:274-324): orthogonal rotations
+    leave q.k unchanged, so the output must stay close to unquantised attention."""
+    from mindiesd.quantization import FP8RotateQuantFA
+    from oracle.attention import attention_math
+    g = torch.Generator().manual_seed(9)
+    rot_q, _ = torch.linalg.qr(torch.randn(128, 128, generator=g))
+    weights = {"blk.attn.q_rot": rot_q.to(torch.bfloat16).to(cuda), "blk.attn.k_rot": rot_q.to(torch.bfloat16).to(cuda)}
+    mod = FP8RotateQuantFA(prefix="blk.attn", weights=weights)
+    q, k, v = _outlier_inputs((1, 600, 2, 128), seed=11)
+    out = mod(q.to(cuda), k.to(cuda), v.to(cuda), layout="BSND").cpu()
+    ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=False)
+    assert out.shape == q.shape and cosine(out, ref) > 0.995
+    with pytest.raises(ValueError):
+        mod(q.to(cuda), k.to(cuda), v.to(cuda), layout="SBH")
