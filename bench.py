@@ -112,32 +112,32 @@ def median(xs):
 
 
 # ---- CPU baseline -------------------------------------------------------------------------------------
-def cpu_baseline_dense(cfg, target_s=15.0):
-    """The oracle's attention_math (the reference's unfused torch path restated) on one head and a
-    sample of query rows against the full key/value sequence of the benchmark shape; throughput in
-    TFLOP/s over the sample."""
+def cpu_baseline_dense(cfg, target_s=12.0):
+    """The oracle's attention_math (the reference's unfused torch path restated) on single heads of
+    the benchmark shape: blocks of 4096 query rows against the full key/value sequence until about
+    ``target_s`` seconds of CPU work have been timed; throughput in TFLOP/s over that sample."""
     import torch
     from oracle.attention import attention_math_rows
     g = torch.Generator().manual_seed(0)
     s, d = cfg["S"], cfg["D"]
     k = (torch.randn(1, 1, s, d, generator=g) * 0.5).to(torch.bfloat16)
     v = (torch.randn(1, 1, s, d, generator=g) * 0.5).to(torch.bfloat16)
-    rows = 256
-    q = (torch.randn(1, 1, rows, d, generator=g) * 0.5).to(torch.bfloat16)
-    t0 = time.perf_counter()
-    attention_math_rows(q, k, v, d ** -0.5, row_chunk=256)
-    probe = time.perf_counter() - t0
-    rows = int(min(s, max(256, 256 * round(target_s / max(probe, 1e-3)))))
-    rows = min(rows, 8192)
-    q = (torch.randn(1, 1, rows, d, generator=g) * 0.5).to(torch.bfloat16)
-    t0 = time.perf_counter()
-    attention_math_rows(q, k, v, d ** -0.5, row_chunk=256)
-    dt = time.perf_counter() - t0
+    rows_blk = 4096
+    q = (torch.randn(1, 1, rows_blk, d, generator=g) * 0.5).to(torch.bfloat16)
+    attention_math_rows(q[:, :, :256], k, v, d ** -0.5, row_chunk=256)   # warm the thread pool
+    rows, t0 = 0, time.perf_counter()
+    while True:
+        attention_math_rows(q, k, v, d ** -0.5, row_chunk=512)
+        rows += rows_blk
+        dt = time.perf_counter() - t0
+        if dt >= target_s or rows >= 40 * s:
+            break
     flops = 4.0 * rows * s * d
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"oracle attention_math, 1 head, {rows} query rows x {s} keys of the benchmark shape, "
-                  f"{dt:.1f} s on {os.cpu_count()} visible CPUs (torch threads {torch.get_num_threads()})",
+        "sample": f"oracle attention_math, one head at a time, {rows} query rows x {s} keys of the benchmark shape "
+                  f"({rows / s:.2f} heads of 40), {dt:.1f} s on {os.cpu_count()} visible CPUs "
+                  f"(torch threads {torch.get_num_threads()})",
     }
 
 
@@ -190,6 +190,73 @@ def extra_sparse(device, steps, warmup, dense_ms):
     }
 
 
+def outlier_inputs(cfg, device, seed=0, dtype=None):
+    """q, k, v = N(0,1) with 1 % of the elements (seeded Bernoulli) scaled by 8, BNSD."""
+    import torch
+    dtype = dtype or torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(seed)
+    shape = (cfg["B"], cfg["N"], cfg["S"], cfg["D"])
+    outs = []
+    for _ in range(3):
+        x = torch.randn(shape, generator=g, device=device)
+        m = torch.rand(shape, generator=g, device=device) < 0.01
+        outs.append(torch.where(m, x * 8, x).to(dtype))
+    return tuple(outs)
+
+
+def extra_fp8(device, steps, warmup):
+    """FP8 attention at the Wan2.1-14B 480p shape vs the bf16 kernel on the same inputs."""
+    import torch
+    import mindiesd
+    from mindiesd.layers.quant import fp8_attention as f8
+    from mindiesd.layers.quant.block_quant import _block_quant
+    cfg = CFG_14B_480P
+    q, k, v = outlier_inputs(cfg, device, seed=4)
+    scale = cfg["D"] ** -0.5
+    bf16_ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)
+    e2e_ms, _ = time_steps(lambda: f8.fp8_attention_forward(q, k, v), steps, warmup)
+    quant = lambda: (_block_quant(q, 128, "BNSD"), _block_quant(k, 128, "BNSD"), f8.quantize_v_per_channel(v))
+    (q8, qs), (k8, ks), (v8t, vs) = quant()
+    quant_ms, _ = time_steps(quant, steps, warmup)
+    kern_ms, _ = time_steps(lambda: f8.fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale), steps, warmup)
+    out8 = f8.fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale)
+    out16 = mindiesd.attention_forward(q, k, v, head_first=True)
+    cos = float(torch.nn.functional.cosine_similarity(out8.float().flatten(), out16.float().flatten(), dim=0))
+    f = attn_flops(cfg)
+    bm, km, qm, em = median(bf16_ms), median(kern_ms), median(quant_ms), median(e2e_ms)
+    # quantisation pass: read q, k once and v twice (maximum, then quantise), write one byte per element
+    quant_bytes = (4 * 2 + 3 * 1) * cfg["N"] * cfg["S"] * cfg["D"]
+    return {"workload": "FP8 attention B1 N40 S32760 D128, N(0,1) with 1% x8 outliers; Q,K per-128-token scales, "
+                        "V per-channel, P e4m3 per tile",
+            "bf16_ms": bm, "bf16_tflops": f / bm / 1e9,
+            "fp8_kernel_ms": km, "fp8_kernel_tflops": f / km / 1e9, "fp8_kernel_frac_of_fp8_peak": f / km / 1e9 / PEAK_FP8_TFLOPS,
+            "fp8_kernel_speedup_vs_bf16": bm / km,
+            "quant_pass_ms": qm, "quant_pass_gbs": quant_bytes / qm / 1e6,
+            "fp8_end_to_end_ms": em, "fp8_end_to_end_speedup_vs_bf16": bm / em,
+            "cosine_fp8_vs_bf16_kernel": cos}
+
+
+def extra_gemm(device, steps, warmup):
+    """MXFP8 GEMM + SwiGLU of the DiT FFN up-projection."""
+    import torch
+    from mindiesd.layers.quant import mx_quantize, mxfp8_matmul
+    m, k, f = CFG_FFN["M"], CFG_FFN["K"], CFG_FFN["N"]
+    g = torch.Generator(device=device).manual_seed(5)
+    x = torch.randn((m, k), generator=g, device=device).to(torch.bfloat16)
+    w = (torch.randn((2 * f, k), generator=g, device=device) * 0.02).to(torch.bfloat16)
+    wq, ws = mx_quantize(w)
+    del w
+    xq, xs = mx_quantize(x)
+    gemm_ms, _ = time_steps(lambda: mxfp8_matmul(xq, xs, wq, ws, None, torch.bfloat16, swiglu=True), steps, warmup)
+    quant_ms, _ = time_steps(lambda: mx_quantize(x), steps, warmup)
+    flops = 2.0 * m * k * 2 * f
+    gm, qm = median(gemm_ms), median(quant_ms)
+    return {"workload": "MXFP8 GEMM + SwiGLU M32760 K5120 N2x13824, x N(0,1), w N(0,0.02)",
+            "gemm_ms": gm, "gemm_tflops": flops / gm / 1e9, "gemm_frac_of_fp8_peak": flops / gm / 1e9 / PEAK_FP8_TFLOPS,
+            "act_quant_ms": qm, "act_quant_gbs": (m * k * 3 + m * k / 32) / qm / 1e6,
+            "with_act_quant_ms": gm + qm}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -197,6 +264,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference kernel for scaling rocprof byte counters)")
+    ap.add_argument("--extras-only", default="",
+                    help="comma separated subset of extras to run (dense_wan1p3b,sparse_rf_v3,fp8_attention,"
+                         "mxfp8_gemm_swiglu)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one GPU's share of the attention path on ONE MI355X; "
@@ -210,6 +282,15 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.calib_copy:
+        src = torch.zeros(1 << 28, dtype=torch.float32, device=device)   # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     cfg = CFG_14B_720P
     q, k, v = dense_inputs(cfg, device, seed=1)
@@ -239,7 +320,11 @@ def main():
     if not args.no_extras:
         extras = {}
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
-                         ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms))):
+                         ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
+                         ("fp8_attention", lambda: extra_fp8(device, args.steps, args.warmup)),
+                         ("mxfp8_gemm_swiglu", lambda: extra_gemm(device, args.steps, args.warmup))):
+            if args.extras_only and name not in args.extras_only.split(","):
+                continue
             try:
                 extras[name] = fn()
             except Exception as e:  # an extra must never cost the main line

@@ -42,6 +42,16 @@ struct Elem<MSD_DTYPE_BF16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ type from_float(float f) { return (__bf16)f; }
+  // acc + sum of the 8 elements (v_dot2_f32_bf16 against ones)
+  static __device__ __forceinline__ float sum8(x8 v, float acc) {
+    typedef __bf16 x2 __attribute__((ext_vector_type(2)));
+    const x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    union { x8 v; x2 p[4]; } u;
+    u.v = v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2_f32_bf16(u.p[i], ones, acc, false);
+    return acc;
+  }
 };
 template <>
 struct Elem<MSD_DTYPE_F16> {
@@ -52,6 +62,15 @@ struct Elem<MSD_DTYPE_F16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ type from_float(float f) { return (_Float16)f; }
+  static __device__ __forceinline__ float sum8(x8 v, float acc) {
+    typedef _Float16 x2 __attribute__((ext_vector_type(2)));
+    const x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    union { x8 v; x2 p[4]; } u;
+    u.v = v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(u.p[i], ones, acc, false);
+    return acc;
+  }
 };
 
 // LDS pointer in address space 3 (needed by the transposing LDS read builtin).

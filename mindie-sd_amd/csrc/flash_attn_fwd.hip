@@ -20,6 +20,8 @@
 // LDS layouts (bank-conflict free for their readers, no padding):
 //     K tile [key][128]: 16-byte chunk c of row key is stored at chunk c ^ (key & 15)
 //     V tile [key][128]: 64-byte chunk c of row key is stored at chunk c ^ (key & 3)
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace msd {
@@ -44,6 +46,7 @@ struct FaParams {
   int kb_stride;
   int QB;
   const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
+  int map_mode;      // 0: consecutive query tiles of a head share an XCD; 1: linear block order
 };
 
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
   const int total = p.B * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
-  int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
   if (work >= total) return;
   if (SPARSE && p.order) work = p.order[blockIdx.x < total ? blockIdx.x : 0];
   if (SPARSE && p.order && blockIdx.x >= total) return;
@@ -140,16 +143,26 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     for (int ks = 0; ks < 8; ++ks) {
       X8 v = *(const X8*)(src + 16 * ks);
       if (!ok) v = X8{0};
+      // fold softmax scale * log2(e) into Q once (the reference rounds q * scale to the input
+      // type as well, attention_func.py:40), so the scores come out of the MFMA in log2 units
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = E::from_float((float)v[j] * p.scale_log2);
       qf[qb][ks] = v;
     }
   }
 
   f32x16_t oacc[4][C::kNQB];
+  // m_run: reference maximum (log2 units) that l_run and oacc are expressed in; negm holds -m_run
+  // in all 16 accumulator slots of a lane and seeds the score accumulators, so the MFMA chain
+  // delivers s - m directly and the softmax needs no subtraction.
   float m_run[C::kNQB], l_run[C::kNQB];
+  f32x16_t negm[C::kNQB];
 #pragma unroll
   for (int qb = 0; qb < C::kNQB; ++qb) {
-    m_run[qb] = -INFINITY;
+    m_run[qb] = 0.f;
     l_run[qb] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negm[qb][r] = 0.f;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -163,8 +176,31 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   // pc ^ swizzle(row).  The per-lane byte offset inside a tile never changes; the tile position
   // is a scalar offset.  Rows past the end of the sequence are out of the buffer's range and read
   // as zeros (their scores are masked to -inf below).
+  // Sparse: the block ids of the list are fetched 64 at a time (one per lane, the next batch is
+  // requested when the current one comes into use) and handed out with v_readlane, so no memory
+  // access sits between two tiles.
+  int sel_cur = 0, sel_nxt = 0, sel_batch = 0;
+  const int n_blk = SPARSE ? n_tiles / kSub : 0;
+  if (SPARSE) {
+    sel_cur = lane < n_blk ? sel[lane] : 0;
+    sel_nxt = 64 + lane < n_blk ? sel[64 + lane] : 0;
+  }
+  auto sel_advance = [&](int t) {  // call once per tile, before tile_key0(t) / tile_key0(t + 1)
+    const int batch = (t / kSub) >> 6;
+    if (batch != sel_batch) {
+      sel_cur = sel_nxt;
+      sel_batch = batch;
+      const int i = 64 * (batch + 1) + lane;
+      sel_nxt = i < n_blk ? sel[i] : 0;
+    }
+  };
   auto tile_key0 = [&](int t) -> int {
-    if (SPARSE) return sel[t / kSub] * 128 + (t % kSub) * BN;
+    if (SPARSE) {
+      const int blk = t / kSub;
+      const int id = (blk >> 6) == sel_batch ? __builtin_amdgcn_readlane(sel_cur, blk & 63)
+                                             : __builtin_amdgcn_readlane(sel_nxt, blk & 63);
+      return id * 128 + (t % kSub) * BN;
+    }
     return t * BN;
   };
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -201,8 +237,11 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; ++t) {
-    const int stage = t & 1;
+  // One tile step.  The LDS stage is a compile-time constant (the loop below is unrolled by two),
+  // so every operand read is `lane-constant register + immediate offset`.
+  auto tile_step = [&](const int t, auto stage_c) {
+    constexpr int stage = decltype(stage_c)::value;
+    if (SPARSE) sel_advance(t);
     if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
 
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
@@ -210,12 +249,6 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 
     // ---- S^T = K Q^T: kNKB independent accumulation chains per 16-wide step of head_dim -------
     f32x16_t sacc[C::kNKB][C::kNQB];
-#pragma unroll
-    for (int kb = 0; kb < C::kNKB; ++kb)
-#pragma unroll
-      for (int qb = 0; qb < C::kNQB; ++qb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kb][qb][r] = 0.f;
     X8 afrag[2][C::kNKB];
 #pragma unroll
     for (int kb = 0; kb < C::kNKB; ++kb)
@@ -232,7 +265,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int qb = 0; qb < C::kNQB; ++qb)
-          sacc[kb][qb] = E::mfma32(afrag[ks & 1][kb], qf[qb][ks], sacc[kb][qb]);
+          sacc[kb][qb] = E::mfma32(afrag[ks & 1][kb], qf[qb][ks], ks == 0 ? negm[qb] : sacc[kb][qb]);
     }
     if (SCHED == 1) {
       // operand reads run one head_dim step ahead of the matrix instructions that consume them
@@ -261,10 +294,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         }
     }
 
-    // ---- online softmax in the exp2 domain with a lazily updated reference maximum --------------
-    // m_run is the reference (scaled by scale*log2 e) that the running sum and the accumulator are
-    // expressed in.  It only moves when some row's new maximum exceeds it by more than kTau, so
-    // the accumulator rescale is skipped for almost every tile; probabilities stay <= 2^kTau.
+    // ---- online softmax in the exp2 domain with a lazily moved reference maximum ------------------
+    // sacc already holds s - m_run.  The reference only moves when some row of this tile exceeds
+    // it by more than kTau (or on the first tile), so the exponentials need no per-element
+    // subtraction and the accumulator rescale is skipped for almost every tile; probabilities stay
+    // <= 2^kTau.  Row sums are taken from the rounded probabilities (the values the second product
+    // uses) with a packed dot product against ones.
     X8 pf[C::kNQB][C::kNKB][2];
 #pragma unroll
     for (int qb = 0; qb < C::kNQB; ++qb) {
@@ -273,33 +308,35 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][qb][r]);
-      mx = half_max(mx) * p.scale_log2;
-      if (__builtin_amdgcn_ballot_w64(mx > m_run[qb] + kTau) != 0) {
-        const float m_new = fmaxf(m_run[qb], mx);
-        const float alpha = fast_exp2(m_run[qb] - (m_new == -INFINITY ? 0.f : m_new));
-        m_run[qb] = m_new;
+      mx = half_max(mx);
+      if (t == 0 || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+        // t == 0: move to the exact row maximum (delta may be negative); later: only upwards
+        float delta = (t == 0) ? mx : fmaxf(mx, 0.f);
+        delta = (delta == -INFINITY) ? 0.f : delta;
+        const float alpha = fast_exp2(-delta);
+        m_run[qb] += delta;
         l_run[qb] *= alpha;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) negm[qb][r] = -m_run[qb];
+#pragma unroll
+        for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[kb][qb][r] -= delta;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
           for (int r = 0; r < 16; ++r) oacc[db][qb][r] *= alpha;
       }
-      const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
       float ls = 0.f;
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = fast_exp2(__builtin_fmaf(sacc[kb][qb][r], p.scale_log2, -mc));
-          ls += e;
-          sacc[kb][qb][r] = e;
-        }
-#pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
           X8 pk;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pk[j] = E::from_float(sacc[kb][qb][8 * t2 + j]);
+          for (int j = 0; j < 8; ++j) pk[j] = E::from_float(fast_exp2(sacc[kb][qb][8 * t2 + j]));
           pf[qb][kb][t2] = pk;
+          ls = E::sum8(pk, ls);
         }
       }
       l_run[qb] += ls;
@@ -328,6 +365,10 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): next tile's LDS-DMA issued by this wave is complete
     __syncthreads();
+  };
+  for (int t = 0; t < n_tiles; t += 2) {
+    tile_step(t, std::integral_constant<int, 0>{});
+    if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
   }
 
   // ---- epilogue: normalise, transpose 32 query rows at a time through LDS, coalesced store -------
@@ -373,17 +414,268 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// ---- ping-pong variant (dense) ---------------------------------------------------------------------------
+// Same tiling as fa_fwd_kernel<8 waves x 32 rows, 128-key tiles>, but the two waves that share a SIMD
+// run half an interval apart: between two workgroup barriers, waves 0-3 issue their matrix work
+// (O += P(t) V(t), then S(t+1) = K(t+1) Q^T) and afterwards the softmax of tile t+1, while waves 4-7
+// first run the softmax of tile t and then the same matrix work.  While one wave of a SIMD feeds the
+// matrix pipe the other one keeps the vector ALU busy, instead of both waiting for each other as
+// they do when every wave walks QK^T -> softmax -> PV in lockstep.
+// LDS holds V(t) and K(t+1) for the current interval and receives V(t+1), K(t+2) by LDS-DMA.
+template <int DT>
+__global__ __launch_bounds__(512, 2) void fa_fwd_pp_kernel(const FaParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using E = Elem<DT>;
+  using T = typename E::type;
+  using X8 = typename E::x8;
+  constexpr int NWAVES = 8, BM = 256, BN = 128, kRowBytes = 256;
+  constexpr int kTileBytes = BN * kRowBytes;  // 32 KiB
+  constexpr int kORowBytes = kRowBytes + 8;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  MSD_LDS char* smem = (MSD_LDS char*)smem_raw;  // [K0 | K1 | V0 | V1]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int h = lane >> 5;
+  const bool late = wave >= 4;  // waves 4-7: softmax first, then matrix work
+
+  const int q_tiles = (p.Sq + BM - 1) / BM;
+  const int total = p.B * p.N * q_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
+  if (work >= total) return;
+  const int bn = work / q_tiles;
+  const int qt = work - bn * q_tiles;
+  const int b = bn / p.N;
+  const int n = bn - b * p.N;
+  const int nkv = n / (p.N / p.Nkv);
+  const int q0 = qt * BM;
+  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
+  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
+  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
+  const int n_tiles = (p.Skv + BN - 1) / BN;
+
+  X8 qf[8];
+  {
+    const int qrow = q0 + wave * 32 + l32;
+    const bool ok = qrow < p.Sq;
+    const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * h;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      X8 v = *(const X8*)(src + 16 * ks);
+      if (!ok) v = X8{0};
+      qf[ks] = v;
+    }
+  }
+  f32x16_t oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // ---- LDS-DMA: 4 groups of 4 rows per wave and tile --------------------------------------------------
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)kg, 0, (int)(((long long)(p.Skv - 1) * p.k_ss + 128) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)vg, 0, (int)(((long long)(p.Skv - 1) * p.v_ss + 128) * 2), 0x00020000);
+  const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
+  int k_voff[4], v_voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * (i * NWAVES + wave) + (lane >> 4);
+    const int pc = lane & 15;
+    k_voff[i] = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
+    v_voff[i] = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
+  }
+  auto load_k = [&](int t) {
+    MSD_LDS char* dst = smem + (t & 1) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(dst + (i * NWAVES + wave) * 1024), 16, k_voff[i],
+                                               t * BN * k_row_bytes, 0, 0);
+  };
+  auto load_v = [&](int t) {
+    MSD_LDS char* dst = smem + (2 + (t & 1)) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(dst + (i * NWAVES + wave) * 1024), 16, v_voff[i],
+                                               t * BN * v_row_bytes, 0, 0);
+  };
+
+  const int k_row_off = l32 * kRowBytes;
+  const int k_swz = l32 & 15;
+  const int v_key = 4 * h + ((lane & 15) >> 2);
+  const int v_row_off = v_key * kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+  const int v_swz = (lane & 15) >> 2;
+
+  f32x16_t sacc[4];
+  X8 pf[4][2];
+
+  // S^T(t) = K(t) Q^T
+  auto qk = [&](int t) {
+    MSD_LDS const char* kb_base = smem + (t & 1) * kTileBytes;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+    X8 afrag[2][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+      afrag[0][kb] = *(MSD_LDS const X8*)(kb_base + kb * 32 * kRowBytes + k_row_off + ((h ^ k_swz) << 4));
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks + 1 < 8) {
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+          afrag[(ks + 1) & 1][kb] =
+              *(MSD_LDS const X8*)(kb_base + kb * 32 * kRowBytes + k_row_off + (((2 * (ks + 1) + h) ^ k_swz) << 4));
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) sacc[kb] = E::mfma32(afrag[ks & 1][kb], qf[ks], sacc[kb]);
+    }
+    const int key0 = t * BN;
+    if (key0 + BN > p.Skv) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3) >= p.Skv) sacc[kb][r] = -INFINITY;
+    }
+  };
+  // P^T(t) from S^T(t): online softmax in the exp2 domain with a lazily moved reference maximum
+  auto softmax = [&]() {
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+    mx = half_max(mx) * p.scale_log2;
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
+    const float mc = (m_run == -INFINITY) ? 0.f : m_run;
+    float ls = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = fast_exp2(__builtin_fmaf(sacc[kb][r], p.scale_log2, -mc));
+        ls += e;
+        sacc[kb][r] = e;
+      }
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        X8 pk;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pk[j] = E::from_float(sacc[kb][8 * t2 + j]);
+        pf[kb][t2] = pk;
+      }
+    }
+    l_run += ls;
+  };
+  // O^T += V(t)^T P^T(t)
+  auto pv = [&](int t) {
+    MSD_LDS const char* vb_base = smem + (2 + (t & 1)) * kTileBytes;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          MSD_LDS const char* src = vb_base + (kb * 32 + 16 * t2) * kRowBytes + v_row_off + ((db ^ v_swz) << 6);
+          const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)src);
+          const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)(src + 8 * kRowBytes));
+          union { s16x4_t s[2]; X8 x; } u;
+          u.s[0] = lo;
+          u.s[1] = hi;
+          oacc[db] = E::mfma32(u.x, pf[kb][t2], oacc[db]);
+        }
+  };
+
+  // ---- prologue: K(0), V(0), K(1) in LDS; S(0) for everybody, P(0) for the early waves ----------------
+  load_k(0);
+  load_v(0);
+  if (n_tiles > 1) load_k(1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+  qk(0);
+  if (!late) softmax();
+
+  for (int t = 0; t < n_tiles; ++t) {
+    // interval t: V(t) and K(t+1) are in LDS; fetch V(t+1) and K(t+2) for the next interval
+    if (t + 1 < n_tiles) load_v(t + 1);
+    if (t + 2 < n_tiles) load_k(t + 2);
+    if (late) softmax();
+    pv(t);
+    if (t + 1 < n_tiles) {
+      qk(t + 1);
+      if (!late) softmax();
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------
+  MSD_LDS char* ost = smem + wave * 32 * kORowBytes;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+  const float l_tot = half_sum(l_run);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const int qrow_l = q0 + wave * 32 + l32;
+  if (p.lse && h == 0 && qrow_l < p.Sq) {
+    const long long li = ((long long)b * p.N + n) * p.Sq + qrow_l;
+    p.lse[li] = l_tot > 0.f ? m_run * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
+  }
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      typename E::x4 pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[j] = E::from_float(oacc[db][4 * g + j] * inv);
+      const int d = db * 32 + 8 * g + 4 * h;
+      *(MSD_LDS typename E::x4*)(ost + l32 * kORowBytes + d * 2) = pk;
+    }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = i * 64 + lane;
+    const int row = c >> 4, c16 = c & 15;
+    const int qrow = q0 + wave * 32 + row;
+    const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16);
+    const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16 + 8);
+    if (qrow < p.Sq) *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
+  }
+#endif
+}
+
+template <int DT>
+static int launch_fa_pp(const FaParams& p, hipStream_t stream) {
+  constexpr int kLds = 4 * 128 * 256;  // K0 K1 V0 V1
+  auto kern = fa_fwd_pp_kernel<DT>;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+    return MSD_ERR_LAUNCH;
+  const int total = p.B * p.N * ((p.Sq + 255) / 256);
+  hipLaunchKernelGGL(kern, dim3((total + 7) / 8 * 8), dim3(512), kLds, stream, p);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
   auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED>;
-  static bool configured = false;  // raising the dynamic LDS limit is idempotent
-  if (!configured) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) !=
-        hipSuccess)
-      return MSD_ERR_LAUNCH;
-    configured = true;
-  }
+  // per device and idempotent, so it is simply repeated on every launch
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
+    return MSD_ERR_LAUNCH;
   const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
   const int total = p.B * p.N * q_tiles;
   const int grid = ((total + 7) / 8) * 8;
@@ -402,7 +694,11 @@ extern "C" {
 //  1: 4 waves x 32 rows, 64-key tiles, compiler scheduling; 2: as 0 with compiler scheduling;
 //  3: as 1 with scheduled operand reads).
 static int g_dense_variant = 0;
-void mindiesd_set_dense_variant(int v) { g_dense_variant = v; }
+static int g_map_mode = 0;  // bits 8.. of the variant: tile order (0 = per-XCD chunks, 1 = linear)
+void mindiesd_set_dense_variant(int v) {
+  g_dense_variant = v & 0xff;
+  g_map_mode = (v >> 8) & 0xff;
+}
 
 static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
                         int Nkv, int Sq, int Skv, int D, const long long* st, float scale) {
@@ -447,6 +743,7 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
   if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.order = order;
+  p.map_mode = g_map_mode;
   p.QB = (Sq + 127) / 128;
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
@@ -460,9 +757,11 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
   const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
   if (rc != MSD_OK) return rc;
-  const FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  p.map_mode = g_map_mode;
   if (dtype == MSD_DTYPE_BF16) {
     switch (g_dense_variant) {
+      case 4: return launch_fa_pp<MSD_DTYPE_BF16>(p, stream);
       case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);
       case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
       case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);

