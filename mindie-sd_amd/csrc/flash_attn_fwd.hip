@@ -120,17 +120,14 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
   const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
 
-  // ---- tile list ----------------------------------------------------------------------------
-  int n_tiles;
-  const int* sel = nullptr;
-  constexpr int kSub = 128 / BN;  // tiles per 128-key block (sparse granularity)
-  if (SPARSE) {
-    const long long qb_lin = (long long)bn * p.QB + qt;  // BM == 128 for the sparse kernel
-    sel = p.blk_idx + qb_lin * p.kb_stride;
-    n_tiles = p.blk_cnt[qb_lin] * kSub;
-  } else {
-    n_tiles = (p.Skv + BN - 1) / BN;
-  }
+  // ---- tile stream ----------------------------------------------------------------------------
+  // Dense: key tiles 0, BN, 2*BN, ...  Sparse: a workgroup owns kBM/128 query blocks (one per group
+  // of 4 waves); it walks the ascending MERGE of their block lists, every key block is staged in
+  // LDS once, and a wave computes on it only if its own query block selected it.
+  constexpr int kSub = 128 / BN;          // tiles per 128-key block (sparse granularity)
+  constexpr int kQBlocks = C::kBM / 128;  // query blocks per workgroup (sparse)
+  static_assert(!SPARSE || kQBlocks == 1 || kQBlocks == 2, "sparse kernel handles 1 or 2 query blocks");
+  const int grp = SPARSE ? wave / 4 : 0;  // which of the workgroup's query blocks this wave belongs to
 
   // ---- Q^T operand, resident in registers: lane (q = l32, h) holds d = 16*ks + 8*h .. +8 -----
   X8 qf[C::kNQB][8];
@@ -176,33 +173,6 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   // pc ^ swizzle(row).  The per-lane byte offset inside a tile never changes; the tile position
   // is a scalar offset.  Rows past the end of the sequence are out of the buffer's range and read
   // as zeros (their scores are masked to -inf below).
-  // Sparse: the block ids of the list are fetched 64 at a time (one per lane, the next batch is
-  // requested when the current one comes into use) and handed out with v_readlane, so no memory
-  // access sits between two tiles.
-  int sel_cur = 0, sel_nxt = 0, sel_batch = 0;
-  const int n_blk = SPARSE ? n_tiles / kSub : 0;
-  if (SPARSE) {
-    sel_cur = lane < n_blk ? sel[lane] : 0;
-    sel_nxt = 64 + lane < n_blk ? sel[64 + lane] : 0;
-  }
-  auto sel_advance = [&](int t) {  // call once per tile, before tile_key0(t) / tile_key0(t + 1)
-    const int batch = (t / kSub) >> 6;
-    if (batch != sel_batch) {
-      sel_cur = sel_nxt;
-      sel_batch = batch;
-      const int i = 64 * (batch + 1) + lane;
-      sel_nxt = i < n_blk ? sel[i] : 0;
-    }
-  };
-  auto tile_key0 = [&](int t) -> int {
-    if (SPARSE) {
-      const int blk = t / kSub;
-      const int id = (blk >> 6) == sel_batch ? __builtin_amdgcn_readlane(sel_cur, blk & 63)
-                                             : __builtin_amdgcn_readlane(sel_nxt, blk & 63);
-      return id * 128 + (t % kSub) * BN;
-    }
-    return t * BN;
-  };
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)kg, 0, (int)(((long long)(p.Skv - 1) * p.k_ss + C::kD) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -216,8 +186,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     k_voff[i] = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
     v_voff[i] = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
   }
-  auto load_tile = [&](int t, int stage) {
-    const int key0 = tile_key0(t);
+  auto load_tile = [&](int key0, int stage) {
     MSD_LDS char* kb = smem + stage * C::kStageBytes;
     tile_dma<C::kGroupsPerWave, NWAVES>(k_rsrc, v_rsrc, kb, kb + C::kTileBytes, k_voff, v_voff, wave,
                                         key0 * k_row_bytes, key0 * v_row_bytes);
@@ -233,17 +202,81 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int v_row_off = v_key * C::kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
   const int v_swz = (lane & 15) >> 2;
 
-  if (n_tiles > 0) load_tile(0, 0);
+  // ---- stream state (all wave-uniform) -----------------------------------------------------------
+  // Block lists live in registers, 64 ids per batch (one per lane); the next batch is requested when
+  // the current one comes into use and ids are handed out with v_readlane, so no memory access sits
+  // between two tiles.
+  constexpr int kEnd = 0x7fffffff;
+  int l_cur[2] = {0, 0}, l_nxt[2] = {0, 0}, l_pos[2] = {0, 0}, l_n[2] = {0, 0};
+  const int* l_ptr[2] = {nullptr, nullptr};
+  if (SPARSE) {
+#pragma unroll
+    for (int i = 0; i < kQBlocks; ++i) {
+      const int qblk = qt * kQBlocks + i;
+      if (qblk < p.QB) {
+        const long long qb_lin = (long long)bn * p.QB + qblk;
+        l_ptr[i] = p.blk_idx + qb_lin * p.kb_stride;
+        l_n[i] = p.blk_cnt[qb_lin];
+        l_cur[i] = lane < l_n[i] ? l_ptr[i][lane] : 0;
+        l_nxt[i] = 64 + lane < l_n[i] ? l_ptr[i][64 + lane] : 0;
+      }
+    }
+  }
+  auto list_head = [&](int i) -> int {
+    return l_pos[i] < l_n[i] ? __builtin_amdgcn_readlane(l_cur[i], l_pos[i] & 63) : kEnd;
+  };
+  auto list_pop = [&](int i) {
+    ++l_pos[i];
+    if ((l_pos[i] & 63) == 0) {
+      l_cur[i] = l_nxt[i];
+      const int j = l_pos[i] + 64 + lane;
+      l_nxt[i] = j < l_n[i] ? l_ptr[i][j] : 0;
+    }
+  };
+  // cur_*: the tile being computed; nxt_*: the tile being fetched.  key0 < 0 marks the end.
+  int cur_key0 = -1, nxt_key0 = -1, cur_fl = 0, nxt_fl = 0, sub = 0;
+  const int dense_tiles = (p.Skv + BN - 1) / BN;
+  auto stream_next = [&](int& key0, int& fl) {  // sparse: produce the tile after the one produced last
+    if (sub > 0) {  // remaining sub-tiles of the current 128-key block
+      key0 = key0 + BN;
+      sub = (sub + 1) % kSub;
+      return;
+    }
+    const int ka = list_head(0), kb = kQBlocks > 1 ? list_head(1) : kEnd;
+    const int k = ka < kb ? ka : kb;
+    if (k == kEnd) {
+      key0 = -1;
+      fl = 0;
+      return;
+    }
+    fl = (ka == k ? 1 : 0) | (kb == k ? 2 : 0);
+    if (ka == k) list_pop(0);
+    if (kQBlocks > 1 && kb == k) list_pop(1);
+    key0 = k * 128;
+    sub = kSub > 1 ? 1 : 0;
+  };
+  if (SPARSE) {
+    stream_next(cur_key0, cur_fl);
+    nxt_key0 = cur_key0;
+    nxt_fl = cur_fl;
+    if (cur_key0 >= 0) {
+      load_tile(cur_key0, 0);
+      stream_next(nxt_key0, nxt_fl);
+    }
+  } else {
+    load_tile(0, 0);
+  }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
+  bool first = true;  // no tile has been folded into this wave's running softmax yet
 
-  // One tile step.  The LDS stage is a compile-time constant (the loop below is unrolled by two),
-  // so every operand read is `lane-constant register + immediate offset`.
-  auto tile_step = [&](const int t, auto stage_c) {
+  // One tile step: fetch the tile at next_key0 (< 0: none) into the other stage, compute on the tile
+  // at key0 if this wave takes part in it.  The LDS stage is a compile-time constant (the loops
+  // below are unrolled by two), so every operand read is `lane-constant register + immediate offset`.
+  auto tile_step = [&](auto stage_c, const int key0, const int next_key0, const bool active) {
     constexpr int stage = decltype(stage_c)::value;
-    if (SPARSE) sel_advance(t);
-    if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
-
+    if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+    if (active) {
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
     MSD_LDS const char* vb_base = kb_base + C::kTileBytes;
 
@@ -280,7 +313,6 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
 
     // ---- mask keys past the end of the sequence (last tile only) --------------------------------
-    const int key0 = tile_key0(t);
     if (key0 + BN > p.Skv) {
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb)
@@ -309,9 +341,9 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][qb][r]);
       mx = half_max(mx);
-      if (t == 0 || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
-        // t == 0: move to the exact row maximum (delta may be negative); later: only upwards
-        float delta = (t == 0) ? mx : fmaxf(mx, 0.f);
+      if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+        // first tile: move to the exact row maximum (delta may be negative); later: only upwards
+        float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
         const float alpha = fast_exp2(-delta);
         m_run[qb] += delta;
@@ -363,12 +395,30 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       }
     }
 
+      first = false;
+    }  // active
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): next tile's LDS-DMA issued by this wave is complete
     __syncthreads();
   };
-  for (int t = 0; t < n_tiles; t += 2) {
-    tile_step(t, std::integral_constant<int, 0>{});
-    if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
+  if (SPARSE) {
+    // the fetched tile becomes current, the one after it is fetched next
+    auto sparse_step = [&](auto stage_c) {
+      tile_step(stage_c, cur_key0, nxt_key0, ((cur_fl >> grp) & 1) != 0);
+      cur_key0 = nxt_key0;
+      cur_fl = nxt_fl;
+      if (nxt_key0 >= 0) stream_next(nxt_key0, nxt_fl);
+    };
+    while (cur_key0 >= 0) {
+      sparse_step(std::integral_constant<int, 0>{});
+      if (cur_key0 < 0) break;
+      sparse_step(std::integral_constant<int, 1>{});
+    }
+  } else {
+    for (int t = 0; t < dense_tiles; t += 2) {
+      tile_step(std::integral_constant<int, 0>{}, t * BN, t + 1 < dense_tiles ? (t + 1) * BN : -1, true);
+      if (t + 1 < dense_tiles)
+        tile_step(std::integral_constant<int, 1>{}, (t + 1) * BN, t + 2 < dense_tiles ? (t + 2) * BN : -1, true);
+    }
   }
 
   // ---- epilogue: normalise, transpose 32 query rows at a time through LDS, coalesced store -------
@@ -745,6 +795,13 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
   p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.order = order;
   p.map_mode = g_map_mode;
   p.QB = (Sq + 127) / 128;
+  if (g_dense_variant == 7) {
+    // tuning hook: two query blocks per workgroup walking the merge of their lists (128-key tiles).
+    // Pays off only when neighbouring query blocks select mostly the same key blocks.
+    if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, true, 1>(p, stream);
+    return launch_fa<MSD_DTYPE_F16, 8, 32, 128, true, 1>(p, stream);
+  }
+  // one query block per workgroup, 64-key sub-tiles, two workgroups per CU
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
 }

@@ -16,6 +16,8 @@
 //            group of 64 keys the keys are stored in the order in which the S^T accumulator of the
 //            first product hands them to the second one: position 32*h + j holds key
 //            32*(j/16) + 8*((j%16)/4) + 4*h + j%4   (h = 0,1 the wave half, j = 0..31).
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace msd {
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY;
 
   // ---- LDS-DMA staging: one instruction = 8 rows x 128 bytes ----------------------------------------------------
   const unsigned char* kg = p.k8 + (long long)bn * p.Skv * 128;
@@ -288,12 +290,21 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   const int row_off = l32 * 128;
   const int swz = (l32 >> 1) & 7;
 
+  // Row sums come from the matrix core: one extra MFMA per 64 keys with an all-ones A operand
+  // leaves sum_k P8[k][q] in every row of lacc, so the softmax needs no per-element additions and
+  // the denominator is built from exactly the quantised probabilities the numerator uses.
+  f32x16_t lacc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) lacc[r] = 0.f;
+  const i32x8_t ones8 = {0x38383838, 0x38383838, 0x38383838, 0x38383838,
+                         0x38383838, 0x38383838, 0x38383838, 0x38383838};  // E4M3 1.0
+
   if (n_tiles > 0) load_tile(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; ++t) {
-    const int stage = t & 1;
+  auto tile_step = [&](const int t, auto stage_c) {
+    constexpr int stage = decltype(stage_c)::value;
     if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
     MSD_LDS const char* kb_base = smem + stage * kStage;
     MSD_LDS const char* vb_base = kb_base + kTile;
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
           if (key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3) >= p.Skv) sacc[kb][r] = -INFINITY;
     }
 
-    // ---- online softmax (exp2 domain, lazily updated reference maximum), P -> E4M3 ------------------------------
+    // ---- online softmax (exp2 domain, lazily moved reference maximum), P -> E4M3 -------------------------------
     const float c = q_sc * k_sc[t];  // dequantisation scales of this tile folded into the softmax scale
     float mx = sacc[0][0];
 #pragma unroll
@@ -337,33 +348,29 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
       m_run = m_new;
-      l_run *= alpha;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) lacc[r] *= alpha;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
     }
     const float mc = (m_run == -INFINITY ? 0.f : m_run) - kPShift;
-    float ls = 0.f;
     i32x8_t pf[2];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = fast_exp2(__builtin_fmaf(sacc[kb][r], c, -mc));
-        ls += e;
-        sacc[kb][r] = e;
-      }
-#pragma unroll
       for (int g4 = 0; g4 < 4; ++g4)
-        pf[kb >> 1][(kb & 1) * 4 + g4] =
-            pack4_e4m3_noclamp(sacc[kb][4 * g4], sacc[kb][4 * g4 + 1], sacc[kb][4 * g4 + 2], sacc[kb][4 * g4 + 3]);
+        pf[kb >> 1][(kb & 1) * 4 + g4] = pack4_e4m3_noclamp(
+            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4], c, -mc)), fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 1], c, -mc)),
+            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 2], c, -mc)),
+            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 3], c, -mc)));
     }
-    l_run += ls;
 
-    // ---- O^T += V^T P^T (fp8) ---------------------------------------------------------------------------------------
+    // ---- O^T += V^T P^T (fp8), row sums ---------------------------------------------------------------------------
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
+      lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones8, pf[kk], lacc, 0, 0, 0, 0, 0, 0);
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
         MSD_LDS const char* src = vb_base + db * 32 * 128 + row_off;
@@ -376,11 +383,15 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
+  };
+  for (int t = 0; t < n_tiles; t += 2) {
+    tile_step(t, std::integral_constant<int, 0>{});
+    if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
   }
 
   // ---- epilogue: 1/l, per-channel V scale, transpose through LDS, coalesced store -----------------------------------
   // (the 2^kPShift factor is in both the accumulator and the running sum, so it cancels)
-  const float l_tot = half_sum(l_run);
+  const float l_tot = lacc[0];  // every row of lacc holds the full sum over all keys
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const float* vs = p.v_scale + (long long)bn * 128;
   MSD_LDS char* ost = smem + wave * 32 * kORow;
