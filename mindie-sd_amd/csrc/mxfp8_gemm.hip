@@ -85,12 +85,18 @@ struct GemmParams {
   int tiles_m, tiles_n;
 };
 
+// Work decomposition: one workgroup of 4 waves owns a 256 x 256 tile of (X rows) x (W rows); every wave owns
+// 128 x 128 of it as 4 x 4 accumulator blocks (256 accumulator registers, one wave per SIMD), so each
+// 64-wide K step costs 16 KiB of LDS reads per wave for 16 matrix instructions.  K is walked in stages of
+// 64 codes (32 KiB of LDS: X 256 x 64 B, W 256 x 64 B) through a ring of four buffers filled by LDS-DMA:
+// while stage kt is multiplied from registers, stage kt+1 is read from LDS into the other register set,
+// stage kt+2 has just landed and stages kt+3 and kt+4 are in flight.
 template <int DT, bool SWIGLU>
-__global__ __launch_bounds__(512, 2) void mxfp8_gemm_kernel(const GemmParams p) {
+__global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
   using T = typename E::type;
-  constexpr int BM = 256, BNW = 256, BK = 128, NW = 8;
+  constexpr int BM = 256, BNW = 256, BK = 64, NW = 4, NS = 4;
   constexpr int kATile = BM * BK, kWTile = BNW * BK, kStage = kATile + kWTile;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   MSD_LDS char* smem = (MSD_LDS char*)smem_raw;
@@ -115,47 +121,83 @@ __global__ __launch_bounds__(512, 2) void mxfp8_gemm_kernel(const GemmParams p) 
   const int half = p.Nw >> 1;
   const int f0 = SWIGLU ? tn * 128 : tn * 256;
 
-  // ---- LDS-DMA descriptors: one instruction = 8 rows x 128 bytes; 64 instructions per stage, 8 per wave --------
+  // ---- LDS-DMA: one instruction = 16 rows x 64 bytes; 16 + 16 instructions per stage, 4 + 4 per wave ----------
+  // A row keeps its four 16-byte chunks at positions chunk ^ ((row >> 2) & 3), which makes the 16-byte
+  // operand reads of 16 consecutive rows hit 16 different bank groups.
   const __amdgpu_buffer_rsrc_t a_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)min((long long)p.M * p.K, 0x7fffffffll), 0x00020000);
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, (int)min((long long)p.Nw * p.K, 0x7fffffffll), 0x00020000);
+  constexpr int kOutOfRange = 0x7ffffff0;  // lane offset beyond any buffer: the access reads zeros
+  const int k_tiles = p.K / BK;
+  const __amdgpu_buffer_rsrc_t none_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
   int a_voff[4], w_voff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = 8 * (i * NW + wave) + (lane >> 3);  // row inside the 256-row tile
-    const int c = (lane & 7) ^ ((row >> 1) & 7);
+    const int row = 16 * (i * NW + wave) + (lane >> 2);  // row inside the 256-row tile
+    const int c = (lane & 3) ^ ((row >> 2) & 3);
     a_voff[i] = (m0 + row) * p.K + c * 16;  // rows past M are out of range and read as zeros
     int wrow;
     if (SWIGLU) wrow = row < 128 ? f0 + row : half + f0 + (row - 128);
     else wrow = f0 + row;
     // rows past the matrix (or past the gate half) must not alias other rows: push them out of range
     const bool w_ok = SWIGLU ? (f0 + (row & 127) < half) : (wrow < p.Nw);
-    w_voff[i] = w_ok ? wrow * p.K + c * 16 : 0x7ffffff0;
+    w_voff[i] = w_ok ? wrow * p.K + c * 16 : kOutOfRange;
   }
-  auto load_tile = [&](int kt, int stage) {
-    MSD_LDS char* ab = smem + stage * kStage;
+  // Stages past the end of K are requested through an empty descriptor: the DMA then writes zeros and
+  // costs no memory traffic, which keeps the number of outstanding operations the same in every iteration.
+  auto load_stage = [&](int kt, int buf) {
+    MSD_LDS char* ab = smem + buf * kStage;
+    const bool valid = kt < k_tiles;
+    const __amdgpu_buffer_rsrc_t ar = valid ? a_rsrc : none_rsrc;
+    const __amdgpu_buffer_rsrc_t wr = valid ? w_rsrc : none_rsrc;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int g = i * NW + wave;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (MSD_LDS void*)(ab + g * 1024), 16, a_voff[i], kt * BK, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (MSD_LDS void*)(ab + kATile + g * 1024), 16, w_voff[i], kt * BK, 0,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (MSD_LDS void*)(ab + g * 1024), 16, a_voff[i], kt * BK, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (MSD_LDS void*)(ab + kATile + g * 1024), 16, w_voff[i], kt * BK, 0,
                                                0);
     }
   };
 
-  // ---- scales: one dword (4 MX blocks = 128 K-values) per row and K tile, straight from global/L2 ------------------
-  // Buffer loads with a constant per-lane offset and a scalar K offset; rows past the matrices read
-  // scale byte 0 (2^-127) against all-zero data, which contributes exactly 0.
+  // ---- scales: staged through LDS in chunks of 8 stages (16 scale bytes = 512 K-values per row) -------------------
+  // One 16-byte DMA per row and chunk instead of one dword per row and stage pair: a scale row is a
+  // 128-byte line per 4096 K-values, so short reads of it cost a full L2 request each.  Rows past the
+  // matrices read zeros (scale 2^-127) against all-zero data, which contributes exactly 0.
   const int kblk_row = p.K >> 5;  // scale bytes per row
   const __amdgpu_buffer_rsrc_t as_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (int)((long long)p.M * kblk_row), 0x00020000);
   const __amdgpu_buffer_rsrc_t ws_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.ws, 0, (int)((long long)p.Nw * kblk_row), 0x00020000);
-  int as_off[2], ws_off[4];
+  constexpr int kScBase = NS * kStage, kScBuf = 2 * 256 * 16;  // two chunk buffers: [X rows | W rows] x 16 B
+  int as_voff, ws_voff;
+  {
+    const int row = 64 * wave + lane;  // wave w stages rows 64w .. 64w+63 of both operands
+    as_voff = (m0 + row) * kblk_row;
+    int wrow;
+    if (SWIGLU) wrow = row < 128 ? f0 + row : half + f0 + (row - 128);
+    else wrow = f0 + row;
+    const bool w_ok = SWIGLU ? (f0 + (row & 127) < half) : (wrow < p.Nw);
+    ws_voff = w_ok ? wrow * kblk_row : kOutOfRange;
+  }
+  // Requested at the end of every fourth stage so that the number of outstanding operations repeats with
+  // the ring; the request that falls in the middle of a chunk (or past the end of K) goes through the
+  // empty descriptor into a scrap area and costs nothing.
+  auto load_scale_chunk = [&](int kt_next) {  // kt_next: multiple of 4; the chunk starts at stage kt_next + 4
+    const int chunk = __builtin_amdgcn_readfirstlane((kt_next + 4) >> 3);
+    const bool real = ((kt_next + 4) & 7) == 0 && kt_next + 4 < k_tiles;
+    const __amdgpu_buffer_rsrc_t ar = real ? as_rsrc : none_rsrc;
+    const __amdgpu_buffer_rsrc_t wr = real ? ws_rsrc : none_rsrc;
+    const int dst = __builtin_amdgcn_readfirstlane(real ? kScBase + (chunk & 1) * kScBuf + wave * 1024
+                                                        : kScBase + 2 * kScBuf);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (MSD_LDS void*)(smem + dst), 16, as_voff, chunk * 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (MSD_LDS void*)(smem + dst + (real ? 4096 : 0)), 16, ws_voff,
+                                             chunk * 16, 0, 0);
+  };
   bool w_okk[4];
+  int as_lds[4], ws_lds[4];  // LDS offsets of the lane's scale rows inside a chunk buffer
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) as_off[mb] = (m0 + wm * 64 + mb * 32 + l32) * kblk_row;
+  for (int mb = 0; mb < 4; ++mb) as_lds[mb] = kScBase + (wm * 128 + mb * 32 + l32) * 16;
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     // wave column range: SwiGLU: gate cols wn*64 + {0,32}, up cols the same; plain: wn*128 + nb*32
@@ -163,90 +205,136 @@ __global__ __launch_bounds__(512, 2) void mxfp8_gemm_kernel(const GemmParams p) 
     if (SWIGLU) wrow = (nb < 2 ? 0 : half) + f0 + wn * 64 + (nb & 1) * 32 + l32;
     else wrow = f0 + wn * 128 + nb * 32 + l32;
     w_okk[nb] = SWIGLU ? (f0 + wn * 64 + (nb & 1) * 32 + l32 < half) : (wrow < p.Nw);
-    ws_off[nb] = w_okk[nb] ? wrow * kblk_row : 0x7ffffff0;
+    const int lrow = SWIGLU ? ((nb < 2 ? 0 : 128) + wn * 64 + (nb & 1) * 32 + l32) : (wn * 128 + nb * 32 + l32);
+    ws_lds[nb] = kScBase + 4096 + lrow * 16;
   }
-
-  f32x16_t acc[2][4];
+  struct Scales {
+    int a[4], w[4];
+  };
+  // dword of stage pair `pair` (two stages = 128 K-values = 4 MX blocks)
+  auto read_scales = [&](int pair, Scales& s) {
+    const int off = ((pair >> 2) & 1) * kScBuf + (pair & 3) * 4;
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < 4; ++mb) s.a[mb] = *(MSD_LDS const int*)(smem + as_lds[mb] + off);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) s.w[nb] = *(MSD_LDS const int*)(smem + ws_lds[nb] + off);
+  };
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
 
-  const int k_tiles = p.K / BK;
-  const int swz = (l32 >> 1) & 7;
+  const int swz = (l32 >> 2) & 3;
   const int sh = 8 * h;  // the lane's MX block inside a 64-wide K step is block h
-  // LDS row of this lane inside the stage: A rows wm*64 + mb*32 + l32; W rows (tile-local)
-  int a_row_off[2], w_row_off[4];
+  // LDS offsets of this lane's two operand chunks (MX block 0: chunk h, MX block 1: chunk 2 + h)
+  const int c_lo = (h ^ swz) << 4, c_hi = ((2 + h) ^ swz) << 4;
+  int a_row_off[4], w_row_off[4];
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) a_row_off[mb] = (wm * 64 + mb * 32 + l32) * BK;
+  for (int mb = 0; mb < 4; ++mb) a_row_off[mb] = (wm * 128 + mb * 32 + l32) * BK;
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     const int lrow = SWIGLU ? ((nb < 2 ? 0 : 128) + wn * 64 + (nb & 1) * 32 + l32) : (wn * 128 + nb * 32 + l32);
     w_row_off[nb] = kATile + lrow * BK;
   }
-
-  load_tile(0, 0);
-  int a_sc[2], w_sc[4];
+  struct Frags {
+    i32x8_t a[4], w[4];
+  };
+  auto read_frags = [&](int buf, Frags& f) {
+    MSD_LDS const char* base = smem + buf * kStage;
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) a_sc[mb] = __builtin_amdgcn_raw_buffer_load_b32(as_rsrc, as_off[mb], 0, 0);
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb) w_sc[nb] = __builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, ws_off[nb], 0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);
-  __syncthreads();
-
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int stage = kt & 1;
-    int a_sc_n[2] = {0, 0}, w_sc_n[4] = {0, 0, 0, 0};
-    if (kt + 1 < k_tiles) {
-      load_tile(kt + 1, stage ^ 1);
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) a_sc_n[mb] = __builtin_amdgcn_raw_buffer_load_b32(as_rsrc, as_off[mb], (kt + 1) * 4, 0);
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) w_sc_n[nb] = __builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, ws_off[nb], (kt + 1) * 4, 0);
-    }
-    MSD_LDS const char* base = smem + stage * kStage;
-    // move the lane's scale bytes (block h of K step 0, block 2 + h of K step 1) to bytes 0 and 2
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) a_sc[mb] = (int)((unsigned)a_sc[mb] >> sh);
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) w_sc[nb] = (int)((unsigned)w_sc[nb] >> sh);
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      i32x8_t af[2];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + (((4 * ks + h) ^ swz) << 4));
-        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + (((4 * ks + 2 + h) ^ swz) << 4));
-        af[mb] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + (((4 * ks + h) ^ swz) << 4));
-        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + (((4 * ks + 2 + h) ^ swz) << 4));
-        const i32x8_t wf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-          if (ks == 0)
-            acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mb], wf, acc[mb][nb], 0, 0, 0, a_sc[mb], 0,
-                                                                          w_sc[nb]);
-          else
-            acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mb], wf, acc[mb][nb], 0, 0, 2, a_sc[mb], 2,
-                                                                          w_sc[nb]);
-        }
-      }
+    for (int mb = 0; mb < 4; ++mb) {
+      const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + c_lo);
+      const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + c_hi);
+      f.a[mb] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) a_sc[mb] = a_sc_n[mb];
+    for (int nb = 0; nb < 4; ++nb) {
+      const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + c_lo);
+      const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + c_hi);
+      f.w[nb] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  };
+
+  // Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for every DMA in
+  // flight, the explicit counts below wait only for the stage that is needed.  The empty asm statements
+  // keep the compiler from moving LDS accesses across the barrier.
+  auto wg_barrier = [] {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  // s_waitcnt immediates: vmcnt in bits 3:0 (+ 15:14), lgkmcnt(0) unless noted
+  constexpr int kWaitVm16 = 0x4070, kWaitVm18 = 0x4072;
+  constexpr int kWaitVm24Only = 0x4f78;  // vmcnt(24), LDS reads not waited for
+
+  // ---- prologue: the same issue order the main loop produces, so its wait counts apply from stage 0 -----------
+  // Per wave a stage is 8 DMA instructions and a scale chunk is 2.
+  Scales sc, sn;
+  load_scale_chunk(-4);
+  load_stage(0, 0);
+  load_stage(1, 1);
+  load_stage(2, 2);
+  load_stage(3, 3);
+  __builtin_amdgcn_s_waitcnt(kWaitVm24Only);  // scale chunk 0 and stage 0 landed
+  wg_barrier();
+  Frags fr[2];
+  read_frags(0, fr[0]);
+  read_scales(0, sn);
+  __builtin_amdgcn_s_waitcnt(kWaitVm16);  // stage 1 landed, stage 0 is in registers
+  wg_barrier();
+  load_stage(4, 0);
+
+  // ---- main loop, unrolled over the ring so buffers, register sets, scale selectors and wait counts are
+  // static.  The stage count is rounded up to a multiple of four; the extra stages multiply zeros.
+  auto stage_step = [&](int kt, auto j_c) {
+    constexpr int J = decltype(j_c)::value;   // kt % 4
+    constexpr int CUR = J & 1, NXT = CUR ^ 1;
+    constexpr int OPSEL = (J & 1) ? 2 : 0;    // odd stages use scale bytes 2 and 3 of the pair's dword
+    // nothing moves across a stage boundary
+    __builtin_amdgcn_sched_barrier(0);
+    if ((J & 1) == 0) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) w_sc[nb] = w_sc_n[nb];
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
+      for (int i = 0; i < 4; ++i) {
+        sc.a[i] = (int)((unsigned)sn.a[i] >> sh);
+        sc.w[i] = (int)((unsigned)sn.w[i] >> sh);
+      }
+    }
+    read_frags((J + 1) % NS, fr[NXT]);
+    if (J & 1) read_scales((kt + 1) >> 1, sn);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+        acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fr[CUR].a[mb], fr[CUR].w[nb], acc[mb][nb], 0, 0,
+                                                                      OPSEL, sc.a[mb], OPSEL, sc.w[nb]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+    }
+    // stage kt+2 must have landed (mine: the wait; everybody's: the barrier), and every wave must be done
+    // reading the buffer of stage kt+1 before it is refilled with stage kt+5.  Outstanding after stage
+    // kt+2: stages kt+3 and kt+4, plus the two scale requests made at the end of every fourth stage.
+    __builtin_amdgcn_s_waitcnt((J == 1 || J == 2) ? kWaitVm18 : kWaitVm16);
+    wg_barrier();
+    if (J == 0) load_scale_chunk(kt);
+    load_stage(kt + 5, (J + 1) % NS);
+  };
+  for (int kt = 0; kt < k_tiles; kt += 4) {
+    stage_step(kt, std::integral_constant<int, 0>{});
+    stage_step(kt + 1, std::integral_constant<int, 1>{});
+    stage_step(kt + 2, std::integral_constant<int, 2>{});
+    stage_step(kt + 3, std::integral_constant<int, 3>{});
   }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // the trailing (empty) DMA requests
+  __syncthreads();  // the staging below reuses the ring
 
   // ---- epilogue: bias, SwiGLU, 16-bit, transpose through LDS, coalesced rows -------------------------------------
-  // accumulator (mb, nb): row m = wm*64 + mb*32 + 8*(r/4) + 4*h + r%4, column = l32 of block nb
+  // accumulator (mb, nb): row m = wm*128 + mb*32 + 8*(r/4) + 4*h + r%4, column = l32 of block nb
   constexpr int kOutCols = SWIGLU ? 64 : 128;          // output columns per wave
   constexpr int kORow = kOutCols * 2 + 8;              // padded staging row (bytes)
   MSD_LDS char* ost = smem + wave * 32 * kORow;       // 32 rows per wave at a time
@@ -262,7 +350,7 @@ __global__ __launch_bounds__(512, 2) void mxfp8_gemm_kernel(const GemmParams p) 
   const int col0 = SWIGLU ? f0 + wn * 64 : f0 + wn * 128;
   constexpr int kChunks = kOutCols / 8;  // 16-byte chunks per row
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) {
+  for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = 8 * (r >> 2) + 4 * h + (r & 3);
@@ -285,7 +373,7 @@ __global__ __launch_bounds__(512, 2) void mxfp8_gemm_kernel(const GemmParams p) 
     for (int i = 0; i < 32 * kChunks / 64; ++i) {
       const int cidx = i * 64 + lane;
       const int row = cidx / kChunks, c16 = cidx % kChunks;
-      const int m = m0 + wm * 64 + mb * 32 + row;
+      const int m = m0 + wm * 128 + mb * 32 + row;
       const int col = col0 + c16 * 8;
       const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16);
       const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16 + 8);
@@ -338,7 +426,8 @@ int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const
   p.M = M; p.K = K; p.Nw = Nw; p.Nout = swiglu ? Nw / 2 : Nw;
   p.tiles_m = (M + 255) / 256;
   p.tiles_n = swiglu ? (Nw / 2 + 127) / 128 : (Nw + 255) / 256;
-  constexpr int kLds = 2 * (256 * 128 + 256 * 128);  // 128 KiB; the output staging (8 x 32 rows x 264 B) fits inside
+  constexpr int kLds = 4 * (256 * 64 + 256 * 64) + 2 * 8192 + 1024;  // ring of four 32 KiB stages + two scale chunk buffers + scrap;
+                                                             // the output staging (4 x 32 rows x 264 B) reuses the ring
   const int total = p.tiles_m * p.tiles_n;
   const int grid = (total + 7) / 8 * 8;
 #define MSD_LAUNCH_GEMM(DTV, SW)                                                                                   \
@@ -346,7 +435,7 @@ int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const
     auto kern = mxfp8_gemm_kernel<DTV, SW>;                                                                        \
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)    \
       return MSD_ERR_LAUNCH;                                                                                       \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);                                              \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kLds, stream, p);                                              \
   }
   if (out_dtype == MSD_DTYPE_BF16) {
     if (swiglu) MSD_LAUNCH_GEMM(MSD_DTYPE_BF16, true) else MSD_LAUNCH_GEMM(MSD_DTYPE_BF16, false)
