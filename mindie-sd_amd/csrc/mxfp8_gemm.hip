@@ -85,19 +85,24 @@ struct GemmParams {
   int tiles_m, tiles_n;
 };
 
-// Work decomposition: one workgroup of 4 waves owns a 256 x 256 tile of (X rows) x (W rows); every wave owns
-// 128 x 128 of it as 4 x 4 accumulator blocks (256 accumulator registers, one wave per SIMD), so each
-// 64-wide K step costs 16 KiB of LDS reads per wave for 16 matrix instructions.  K is walked in stages of
-// 64 codes (32 KiB of LDS: X 256 x 64 B, W 256 x 64 B) through a ring of four buffers filled by LDS-DMA:
-// while stage kt is multiplied from registers, stage kt+1 is read from LDS into the other register set,
-// stage kt+2 has just landed and stages kt+3 and kt+4 are in flight.
+// Work decomposition: one workgroup of 4 waves (one per SIMD, 256 accumulator registers each) owns a
+// 256 x 256 tile of (X rows) x (W rows), seen as 2 x 2 quadrants of 128 x 128; inside a quadrant every
+// wave owns 64 x 64 (2 x 2 accumulator blocks).  K is walked in blocks of 128 codes.  The unit of LDS
+// traffic is one operand half of one K block: 128 rows x 128 bytes = 16 KiB, so that every DMA
+// instruction moves full 128-byte lines.  Per K block the quadrants are visited in the order
+// (A0,W0) (A1,W0) (A1,W1) (A0,W1): consecutive steps share one operand half, which stays in registers,
+// so every step reads exactly one new unit from LDS into the register set that has just become free
+// (the roles of the two A sets swap from one K block to the next, hence the unrolling over 8 steps).
+// Units are consumed in the order W0 A0 A1 W1 | W0 A0 A1 W1 | ... and travel through a ring of eight LDS
+// slots: during step t unit t+2 goes from LDS into registers, unit t+3 has landed, units t+4 .. t+9 are
+// in flight.
 template <int DT, bool SWIGLU>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
   using T = typename E::type;
-  constexpr int BM = 256, BNW = 256, BK = 64, NW = 4, NS = 4;
-  constexpr int kATile = BM * BK, kWTile = BNW * BK, kStage = kATile + kWTile;
+  constexpr int BM = 256, BK = 128, NW = 4, NU = 8;
+  constexpr int kUnit = 128 * BK;  // 16 KiB
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   MSD_LDS char* smem = (MSD_LDS char*)smem_raw;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -117,75 +122,70 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
   const int tm = gm0 + in_grp % gsz;
   const int tn = in_grp / gsz;
   const int m0 = tm * BM;
-  // W rows of this tile: plain: 256 consecutive rows; SwiGLU: 128 gate rows + the matching 128 up rows
+  // W rows of this tile: plain: 256 consecutive rows; SwiGLU: 128 gate rows (half W0) + the matching 128
+  // up rows (half W1), so both parts of an output element meet in the same lane and register index
   const int half = p.Nw >> 1;
   const int f0 = SWIGLU ? tn * 128 : tn * 256;
 
-  // ---- LDS-DMA: one instruction = 16 rows x 64 bytes; 16 + 16 instructions per stage, 4 + 4 per wave ----------
-  // A row keeps its four 16-byte chunks at positions chunk ^ ((row >> 2) & 3), which makes the 16-byte
-  // operand reads of 16 consecutive rows hit 16 different bank groups.
+  // ---- LDS-DMA: one instruction = 8 rows x 128 bytes; 16 instructions per unit, 4 per wave ---------------------
+  // A row keeps its eight 16-byte chunks at positions chunk ^ ((row >> 1) & 7), which makes the 16-byte
+  // operand reads of 16 consecutive rows hit 16 different bank groups.  Rows past the end of a matrix are
+  // beyond the descriptor's range and read as zeros; gate rows past the gate part read up rows, whose
+  // products land in columns that are never stored.
   const __amdgpu_buffer_rsrc_t a_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)min((long long)p.M * p.K, 0x7fffffffll), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)((long long)p.M * p.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t w_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, (int)min((long long)p.Nw * p.K, 0x7fffffffll), 0x00020000);
-  constexpr int kOutOfRange = 0x7ffffff0;  // lane offset beyond any buffer: the access reads zeros
-  const int k_tiles = p.K / BK;
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, (int)((long long)p.Nw * p.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t none_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
+  const int k_blocks = p.K / BK;
   int a_voff[4], w_voff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = 16 * (i * NW + wave) + (lane >> 2);  // row inside the 256-row tile
-    const int c = (lane & 3) ^ ((row >> 2) & 3);
-    a_voff[i] = (m0 + row) * p.K + c * 16;  // rows past M are out of range and read as zeros
-    int wrow;
-    if (SWIGLU) wrow = row < 128 ? f0 + row : half + f0 + (row - 128);
-    else wrow = f0 + row;
-    // rows past the matrix (or past the gate half) must not alias other rows: push them out of range
-    const bool w_ok = SWIGLU ? (f0 + (row & 127) < half) : (wrow < p.Nw);
-    w_voff[i] = w_ok ? wrow * p.K + c * 16 : kOutOfRange;
+    const int row = 8 * (i * NW + wave) + (lane >> 3);  // row inside the 128-row unit
+    const int c = (lane & 7) ^ ((row >> 1) & 7);
+    a_voff[i] = (m0 + row) * p.K + c * 16;
+    w_voff[i] = (f0 + row) * p.K + c * 16;
   }
-  // Stages past the end of K are requested through an empty descriptor: the DMA then writes zeros and
-  // costs no memory traffic, which keeps the number of outstanding operations the same in every iteration.
-  auto load_stage = [&](int kt, int buf) {
-    MSD_LDS char* ab = smem + buf * kStage;
-    const bool valid = kt < k_tiles;
-    const __amdgpu_buffer_rsrc_t ar = valid ? a_rsrc : none_rsrc;
-    const __amdgpu_buffer_rsrc_t wr = valid ? w_rsrc : none_rsrc;
+  const int a1_off = 128 * p.K;                          // second half of the X rows
+  const int w1_off = (SWIGLU ? half : 128) * p.K;        // second half of the W rows
+  // kind: 0 = W0, 1 = A0, 2 = A1, 3 = W1 (the order of consumption).  K blocks past the end are requested
+  // through an empty descriptor: the DMA then writes zeros and costs no memory traffic, which keeps the
+  // number of outstanding operations the same in every step.
+  auto load_unit = [&](int kb, auto kind_c, int slot) {
+    constexpr int KIND = decltype(kind_c)::value;
+    constexpr bool IS_A = KIND == 1 || KIND == 2, SECOND = KIND >= 2;
+    const bool valid = kb < k_blocks;
+    const __amdgpu_buffer_rsrc_t rs = valid ? (IS_A ? a_rsrc : w_rsrc) : none_rsrc;
+    MSD_LDS char* ub = smem + slot * kUnit;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int g = i * NW + wave;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (MSD_LDS void*)(ab + g * 1024), 16, a_voff[i], kt * BK, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (MSD_LDS void*)(ab + kATile + g * 1024), 16, w_voff[i], kt * BK, 0,
-                                               0);
+      const int vo = (IS_A ? a_voff[i] : w_voff[i]) + (SECOND ? (IS_A ? a1_off : w1_off) : 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MSD_LDS void*)(ub + (i * NW + wave) * 1024), 16, vo, kb * BK, 0, 0);
     }
   };
 
-  // ---- scales: staged through LDS in chunks of 8 stages (16 scale bytes = 512 K-values per row) -------------------
-  // One 16-byte DMA per row and chunk instead of one dword per row and stage pair: a scale row is a
-  // 128-byte line per 4096 K-values, so short reads of it cost a full L2 request each.  Rows past the
-  // matrices read zeros (scale 2^-127) against all-zero data, which contributes exactly 0.
+  // ---- scales: staged through LDS in chunks of 4 K blocks (16 scale bytes = 512 K-values per row) -------------------
+  // One 16-byte DMA per row and chunk: a scale row is a 128-byte line per 4096 K-values, so short reads
+  // of it would cost a full L2 request each.
   const int kblk_row = p.K >> 5;  // scale bytes per row
   const __amdgpu_buffer_rsrc_t as_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (int)((long long)p.M * kblk_row), 0x00020000);
   const __amdgpu_buffer_rsrc_t ws_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.ws, 0, (int)((long long)p.Nw * kblk_row), 0x00020000);
-  constexpr int kScBase = NS * kStage, kScBuf = 2 * 256 * 16;  // two chunk buffers: [X rows | W rows] x 16 B
+  constexpr int kScBase = NU * kUnit, kScBuf = 2 * 256 * 16;  // two chunk buffers: [X rows | W rows] x 16 B
   int as_voff, ws_voff;
   {
     const int row = 64 * wave + lane;  // wave w stages rows 64w .. 64w+63 of both operands
     as_voff = (m0 + row) * kblk_row;
-    int wrow;
-    if (SWIGLU) wrow = row < 128 ? f0 + row : half + f0 + (row - 128);
-    else wrow = f0 + row;
-    const bool w_ok = SWIGLU ? (f0 + (row & 127) < half) : (wrow < p.Nw);
-    ws_voff = w_ok ? wrow * kblk_row : kOutOfRange;
+    const int wrow = row < 128 ? f0 + row : (SWIGLU ? half + f0 + (row - 128) : f0 + row);
+    ws_voff = wrow * kblk_row;
   }
-  // Requested at the end of every fourth stage so that the number of outstanding operations repeats with
-  // the ring; the request that falls in the middle of a chunk (or past the end of K) goes through the
-  // empty descriptor into a scrap area and costs nothing.
-  auto load_scale_chunk = [&](int kt_next) {  // kt_next: multiple of 4; the chunk starts at stage kt_next + 4
-    const int chunk = __builtin_amdgcn_readfirstlane((kt_next + 4) >> 3);
-    const bool real = ((kt_next + 4) & 7) == 0 && kt_next + 4 < k_tiles;
+  // Requested in every eighth step so that the number of outstanding operations repeats with the
+  // unrolled loop; the request that falls in the middle of a chunk (or past the end of K) goes through
+  // the empty descriptor into a scrap area and costs nothing.
+  auto load_scale_chunk = [&](int t) {  // t: multiple of 8; a chunk is requested 16 steps before its first step
+    const int chunk = __builtin_amdgcn_readfirstlane((t + 16) >> 4);
+    const bool real = (t & 15) == 0 && 4 * chunk < k_blocks;
     const __amdgpu_buffer_rsrc_t ar = real ? as_rsrc : none_rsrc;
     const __amdgpu_buffer_rsrc_t wr = real ? ws_rsrc : none_rsrc;
     const int dst = __builtin_amdgcn_readfirstlane(real ? kScBase + (chunk & 1) * kScBuf + wave * 1024
@@ -194,73 +194,58 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (MSD_LDS void*)(smem + dst + (real ? 4096 : 0)), 16, ws_voff,
                                              chunk * 16, 0, 0);
   };
-  bool w_okk[4];
-  int as_lds[4], ws_lds[4];  // LDS offsets of the lane's scale rows inside a chunk buffer
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) as_lds[mb] = kScBase + (wm * 128 + mb * 32 + l32) * 16;
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    // wave column range: SwiGLU: gate cols wn*64 + {0,32}, up cols the same; plain: wn*128 + nb*32
-    int wrow;
-    if (SWIGLU) wrow = (nb < 2 ? 0 : half) + f0 + wn * 64 + (nb & 1) * 32 + l32;
-    else wrow = f0 + wn * 128 + nb * 32 + l32;
-    w_okk[nb] = SWIGLU ? (f0 + wn * 64 + (nb & 1) * 32 + l32 < half) : (wrow < p.Nw);
-    const int lrow = SWIGLU ? ((nb < 2 ? 0 : 128) + wn * 64 + (nb & 1) * 32 + l32) : (wn * 128 + nb * 32 + l32);
-    ws_lds[nb] = kScBase + 4096 + lrow * 16;
-  }
+  // LDS offsets of the lane's scale rows inside a chunk buffer: X rows a*128 + wm*64 + mb*32 + l32,
+  // W rows (tile-local) w*128 + wn*64 + nb*32 + l32
+  const int as_lds = kScBase + (wm * 64 + l32) * 16;
+  const int ws_lds = kScBase + 4096 + (wn * 64 + l32) * 16;
   struct Scales {
-    int a[4], w[4];
+    int a[2][2], w[2][2];  // [half][block]: one dword = the 4 MX blocks of one K block
   };
-  // dword of stage pair `pair` (two stages = 128 K-values = 4 MX blocks)
-  auto read_scales = [&](int pair, Scales& s) {
-    const int off = ((pair >> 2) & 1) * kScBuf + (pair & 3) * 4;
+  auto read_scales = [&](int kb, Scales& s) {
+    const int off = ((kb >> 2) & 1) * kScBuf + (kb & 3) * 4;
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) s.a[mb] = *(MSD_LDS const int*)(smem + as_lds[mb] + off);
+    for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) s.w[nb] = *(MSD_LDS const int*)(smem + ws_lds[nb] + off);
+      for (int blk = 0; blk < 2; ++blk) {
+        s.a[hf][blk] = *(MSD_LDS const int*)(smem + as_lds + off + (hf * 128 + blk * 32) * 16);
+        s.w[hf][blk] = *(MSD_LDS const int*)(smem + ws_lds + off + (hf * 128 + blk * 32) * 16);
+      }
   };
 
-  f32x16_t acc[4][4];
+  f32x16_t acc[2][2][2][2];  // [A half][W half][mb][nb]
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
+  for (int i = 0; i < 16; ++i)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+    for (int r = 0; r < 16; ++r) (&acc[0][0][0][0])[i][r] = 0.f;
 
-  const int swz = (l32 >> 2) & 3;
+  const int swz = (l32 >> 1) & 7;
   const int sh = 8 * h;  // the lane's MX block inside a 64-wide K step is block h
-  // LDS offsets of this lane's two operand chunks (MX block 0: chunk h, MX block 1: chunk 2 + h)
-  const int c_lo = (h ^ swz) << 4, c_hi = ((2 + h) ^ swz) << 4;
-  int a_row_off[4], w_row_off[4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) a_row_off[mb] = (wm * 128 + mb * 32 + l32) * BK;
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    const int lrow = SWIGLU ? ((nb < 2 ? 0 : 128) + wn * 64 + (nb & 1) * 32 + l32) : (wn * 128 + nb * 32 + l32);
-    w_row_off[nb] = kATile + lrow * BK;
-  }
-  struct Frags {
-    i32x8_t a[4], w[4];
+  // operand fragments of one unit: [block][k step]; k step ks takes chunk 4ks + h (MX block 2ks) and
+  // chunk 4ks + 2 + h (MX block 2ks + 1) of the lane's row
+  struct Frag {
+    i32x8_t v[2][2];
   };
-  auto read_frags = [&](int buf, Frags& f) {
-    MSD_LDS const char* base = smem + buf * kStage;
+  int c_off[2][2];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + c_lo);
-      const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + a_row_off[mb] + c_hi);
-      f.a[mb] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
+  for (int ks = 0; ks < 2; ++ks) {
+    c_off[ks][0] = ((4 * ks + h) ^ swz) << 4;
+    c_off[ks][1] = ((4 * ks + 2 + h) ^ swz) << 4;
+  }
+  const int a_row_off = (wm * 64 + l32) * BK, w_row_off = (wn * 64 + l32) * BK;
+  auto read_unit = [&](int slot, Frag& f, bool is_a) {
+    MSD_LDS const char* base = smem + slot * kUnit + (is_a ? a_row_off : w_row_off);
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + c_lo);
-      const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + w_row_off[nb] + c_hi);
-      f.w[nb] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(base + blk * 32 * BK + c_off[ks][0]);
+        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(base + blk * 32 * BK + c_off[ks][1]);
+        f.v[blk][ks] = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
   };
 
   // Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for every DMA in
-  // flight, the explicit counts below wait only for the stage that is needed.  The empty asm statements
+  // flight, the explicit counts below wait only for the unit that is needed.  The empty asm statements
   // keep the compiler from moving LDS accesses across the barrier.
   auto wg_barrier = [] {
     asm volatile("" ::: "memory");
@@ -268,119 +253,148 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
     asm volatile("" ::: "memory");
   };
   // s_waitcnt immediates: vmcnt in bits 3:0 (+ 15:14), lgkmcnt(0) unless noted
-  constexpr int kWaitVm16 = 0x4070, kWaitVm18 = 0x4072;
+  constexpr int kWaitVm20 = 0x4074, kWaitVm24 = 0x4078, kWaitVm26 = 0x407a;
   constexpr int kWaitVm24Only = 0x4f78;  // vmcnt(24), LDS reads not waited for
 
-  // ---- prologue: the same issue order the main loop produces, so its wait counts apply from stage 0 -----------
-  // Per wave a stage is 8 DMA instructions and a scale chunk is 2.
+  // ---- prologue: the same issue order the main loop produces, so its wait counts apply from step 0 -------------
+  // Per wave a unit is 4 DMA instructions and a scale chunk is 2.
+  using IC0 = std::integral_constant<int, 0>;
+  using IC1 = std::integral_constant<int, 1>;
+  using IC2 = std::integral_constant<int, 2>;
+  using IC3 = std::integral_constant<int, 3>;
   Scales sc, sn;
-  load_scale_chunk(-4);
-  load_stage(0, 0);
-  load_stage(1, 1);
-  load_stage(2, 2);
-  load_stage(3, 3);
-  __builtin_amdgcn_s_waitcnt(kWaitVm24Only);  // scale chunk 0 and stage 0 landed
+  load_scale_chunk(-16);
+  load_unit(0, IC0{}, 0);
+  load_unit(0, IC1{}, 1);
+  load_unit(0, IC2{}, 2);
+  load_unit(0, IC3{}, 3);
+  load_unit(1, IC0{}, 4);
+  load_unit(1, IC1{}, 5);
+  load_unit(1, IC2{}, 6);
+  load_unit(1, IC3{}, 7);
+  __builtin_amdgcn_s_waitcnt(kWaitVm24Only);  // scale chunk 0, units 0 and 1 landed
   wg_barrier();
-  Frags fr[2];
-  read_frags(0, fr[0]);
+  Frag fx, fy, fp, fq;  // X rows: fx, fy; W rows: fp, fq
+  read_unit(0, fp, false);
+  read_unit(1, fx, true);
   read_scales(0, sn);
-  __builtin_amdgcn_s_waitcnt(kWaitVm16);  // stage 1 landed, stage 0 is in registers
+  __builtin_amdgcn_s_waitcnt(kWaitVm20);  // unit 2 landed, units 0 and 1 are in registers
   wg_barrier();
-  load_stage(4, 0);
+  load_unit(2, IC0{}, 0);
 
-  // ---- main loop, unrolled over the ring so buffers, register sets, scale selectors and wait counts are
-  // static.  The stage count is rounded up to a multiple of four; the extra stages multiply zeros.
-  auto stage_step = [&](int kt, auto j_c) {
-    constexpr int J = decltype(j_c)::value;   // kt % 4
-    constexpr int CUR = J & 1, NXT = CUR ^ 1;
-    constexpr int OPSEL = (J & 1) ? 2 : 0;    // odd stages use scale bytes 2 and 3 of the pair's dword
-    // nothing moves across a stage boundary
+  // ---- main loop -----------------------------------------------------------------------------------------------------
+  // step t = 4 * kb + q computes quadrant q of K block kb from the register sets (fa, fw), loads unit t+2
+  // from LDS into fl and requests unit t+9 (into the slot of unit t+1, read during the previous step).
+  auto step = [&](int t, auto j_c, const Frag& fa, const Frag& fw, Frag& fl) {
+    constexpr int J = decltype(j_c)::value;  // t % 8
+    constexpr int Q = J & 3;
+    constexpr int AH = (Q == 1 || Q == 2) ? 1 : 0, WH = Q >= 2 ? 1 : 0;
+    constexpr int LKIND = (J + 2) & 3;  // kind of the unit that goes into registers
+    // nothing moves across a step boundary
     __builtin_amdgcn_sched_barrier(0);
-    if ((J & 1) == 0) {
+    if (Q == 0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        sc.a[i] = (int)((unsigned)sn.a[i] >> sh);
-        sc.w[i] = (int)((unsigned)sn.w[i] >> sh);
+        (&sc.a[0][0])[i] = (int)((unsigned)(&sn.a[0][0])[i] >> sh);
+        (&sc.w[0][0])[i] = (int)((unsigned)(&sn.w[0][0])[i] >> sh);
       }
     }
-    read_frags((J + 1) % NS, fr[NXT]);
-    if (J & 1) read_scales((kt + 1) >> 1, sn);
+    if (J == 0) load_scale_chunk(t);
+    load_unit((t + 9) >> 2, std::integral_constant<int, (J + 1) & 3>{}, (J + 1) & 7);
+    read_unit((J + 2) & 7, fl, LKIND == 1 || LKIND == 2);
+    if (Q == 3) read_scales((t >> 2) + 1, sn);
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-        acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fr[CUR].a[mb], fr[CUR].w[nb], acc[mb][nb], 0, 0,
-                                                                      OPSEL, sc.a[mb], OPSEL, sc.w[nb]);
+      for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+        for (int mb = 0; mb < 2; ++mb) {
+          if (ks == 0)
+            acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                fa.v[mb][0], fw.v[nb][0], acc[AH][WH][mb][nb], 0, 0, 0, sc.a[AH][mb], 0, sc.w[WH][nb]);
+          else
+            acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                fa.v[mb][1], fw.v[nb][1], acc[AH][WH][mb][nb], 0, 0, 2, sc.a[AH][mb], 2, sc.w[WH][nb]);
+        }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // one LDS read
+      if (Q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // + one scale read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one matrix instruction
+      if (i & 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);      // one DMA request
+      if (J == 0 && (i == 0 || i == 2)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
     }
-    // stage kt+2 must have landed (mine: the wait; everybody's: the barrier), and every wave must be done
-    // reading the buffer of stage kt+1 before it is refilled with stage kt+5.  Outstanding after stage
-    // kt+2: stages kt+3 and kt+4, plus the two scale requests made at the end of every fourth stage.
-    __builtin_amdgcn_s_waitcnt((J == 1 || J == 2) ? kWaitVm18 : kWaitVm16);
+    // Unit t+3 must have landed (mine: the wait; everybody's: the barrier), and every wave must be done
+    // reading the slot of unit t+2 before the next step refills it.  Requested after unit t+3: six
+    // units, plus the two scale requests of step 0 unless they came before it.
+    __builtin_amdgcn_s_waitcnt(J <= 5 ? kWaitVm26 : kWaitVm24);
     wg_barrier();
-    if (J == 0) load_scale_chunk(kt);
-    load_stage(kt + 5, (J + 1) % NS);
   };
-  for (int kt = 0; kt < k_tiles; kt += 4) {
-    stage_step(kt, std::integral_constant<int, 0>{});
-    stage_step(kt + 1, std::integral_constant<int, 1>{});
-    stage_step(kt + 2, std::integral_constant<int, 2>{});
-    stage_step(kt + 3, std::integral_constant<int, 3>{});
+  const int n_steps = 4 * ((k_blocks + 1) & ~1);  // whole pairs of K blocks; a padding block multiplies zeros
+  for (int t = 0; t < n_steps; t += 8) {
+    step(t + 0, std::integral_constant<int, 0>{}, fx, fp, fy);
+    step(t + 1, std::integral_constant<int, 1>{}, fy, fp, fq);
+    step(t + 2, std::integral_constant<int, 2>{}, fy, fq, fp);
+    step(t + 3, std::integral_constant<int, 3>{}, fx, fq, fy);
+    step(t + 4, std::integral_constant<int, 4>{}, fy, fp, fx);
+    step(t + 5, std::integral_constant<int, 5>{}, fx, fp, fq);
+    step(t + 6, std::integral_constant<int, 6>{}, fx, fq, fp);
+    step(t + 7, std::integral_constant<int, 7>{}, fy, fq, fx);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // the trailing (empty) DMA requests
   __syncthreads();  // the staging below reuses the ring
 
   // ---- epilogue: bias, SwiGLU, 16-bit, transpose through LDS, coalesced rows -------------------------------------
-  // accumulator (mb, nb): row m = wm*128 + mb*32 + 8*(r/4) + 4*h + r%4, column = l32 of block nb
-  constexpr int kOutCols = SWIGLU ? 64 : 128;          // output columns per wave
-  constexpr int kORow = kOutCols * 2 + 8;              // padded staging row (bytes)
+  // accumulator [a][w][mb][nb]: row = a*128 + wm*64 + mb*32 + 8*(r/4) + 4*h + r%4,
+  // W row (tile-local) = w*128 + wn*64 + nb*32 + l32.  Output columns of the wave: SwiGLU: f0 + wn*64 + [0,64)
+  // (gate from w = 0, up from w = 1); plain: f0 + w*128 + wn*64 + [0,64) for w = 0, 1.
+  constexpr int kORow = 64 * 2 + 8;                    // padded staging row (bytes): 64 columns
   MSD_LDS char* ost = smem + wave * 32 * kORow;       // 32 rows per wave at a time
-  float bias_v[4];
+  float bias_v[2][2];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    int wrow;
-    if (SWIGLU) wrow = (nb < 2 ? 0 : half) + f0 + wn * 64 + (nb & 1) * 32 + l32;
-    else wrow = f0 + wn * 128 + nb * 32 + l32;
-    bias_v[nb] = (p.bias && w_okk[nb]) ? p.bias[wrow] : 0.f;
-  }
+  for (int w = 0; w < 2; ++w)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int wrow = (SWIGLU ? w * half : w * 128) + f0 + wn * 64 + nb * 32 + l32;
+      bias_v[w][nb] = (p.bias && wrow < p.Nw) ? p.bias[wrow] : 0.f;
+    }
   T* og = (T*)p.out;
-  const int col0 = SWIGLU ? f0 + wn * 64 : f0 + wn * 128;
-  constexpr int kChunks = kOutCols / 8;  // 16-byte chunks per row
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
+  for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * h + (r & 3);
-      if (SWIGLU) {
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-          const float g = acc[mb][nb][r] + bias_v[nb];
-          const float u = acc[mb][nb + 2][r] + bias_v[nb + 2];
-          const float sg = g * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * g));
-          *(MSD_LDS T*)(ost + row * kORow + (nb * 32 + l32) * 2) = E::from_float(sg * u);
+      for (int w = 0; w < (SWIGLU ? 1 : 2); ++w) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) {
+            float val;
+            if (SWIGLU) {
+              const float g = acc[a][0][mb][nb][r] + bias_v[0][nb];
+              const float u = acc[a][1][mb][nb][r] + bias_v[1][nb];
+              val = g * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * g)) * u;
+            } else {
+              val = acc[a][w][mb][nb][r] + bias_v[w][nb];
+            }
+            *(MSD_LDS T*)(ost + row * kORow + (nb * 32 + l32) * 2) = E::from_float(val);
+          }
         }
-      } else {
+        __builtin_amdgcn_wave_barrier();
+        const int col0 = f0 + (SWIGLU ? 0 : w * 128) + wn * 64;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
-          *(MSD_LDS T*)(ost + row * kORow + (nb * 32 + l32) * 2) = E::from_float(acc[mb][nb][r] + bias_v[nb]);
+        for (int i = 0; i < 4; ++i) {  // 32 rows x 8 chunks of 16 bytes
+          const int cidx = i * 64 + lane;
+          const int row = cidx >> 3, c16 = cidx & 7;
+          const int m = m0 + a * 128 + wm * 64 + mb * 32 + row;
+          const int col = col0 + c16 * 8;
+          const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16);
+          const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16 + 8);
+          if (m < p.M && col < p.Nout) *(i32x4_t*)(og + (long long)m * p.Nout + col) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
+        }
+        __builtin_amdgcn_wave_barrier();
       }
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int i = 0; i < 32 * kChunks / 64; ++i) {
-      const int cidx = i * 64 + lane;
-      const int row = cidx / kChunks, c16 = cidx % kChunks;
-      const int m = m0 + wm * 128 + mb * 32 + row;
-      const int col = col0 + c16 * 8;
-      const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16);
-      const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16 + 8);
-      if (m < p.M && col < p.Nout) *(i32x4_t*)(og + (long long)m * p.Nout + col) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
-    }
-    __builtin_amdgcn_wave_barrier();
-  }
 #endif
 }
 
@@ -418,7 +432,7 @@ int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const
   if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
   if (((uintptr_t)a_scale | (uintptr_t)w_scale) & 3) return MSD_ERR_BAD_ARG;
   // 32-bit buffer offsets
-  if ((long long)M * K >= (1ll << 31) - 1024 || (long long)Nw * K >= (1ll << 31) - 1024) return MSD_ERR_UNSUPPORTED;
+  if ((long long)(M + 256) * K >= (1ll << 31) || (long long)(Nw + 256) * K >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
   GemmParams p{};
   p.a = (const unsigned char*)a; p.as = (const unsigned char*)a_scale;
   p.w = (const unsigned char*)w; p.ws = (const unsigned char*)w_scale;
@@ -426,7 +440,7 @@ int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const
   p.M = M; p.K = K; p.Nw = Nw; p.Nout = swiglu ? Nw / 2 : Nw;
   p.tiles_m = (M + 255) / 256;
   p.tiles_n = swiglu ? (Nw / 2 + 127) / 128 : (Nw + 255) / 256;
-  constexpr int kLds = 4 * (256 * 64 + 256 * 64) + 2 * 8192 + 1024;  // ring of four 32 KiB stages + two scale chunk buffers + scrap;
+  constexpr int kLds = 8 * 16384 + 2 * 8192 + 1024;  // ring of eight 16 KiB units + two scale chunk buffers + scrap;
                                                              // the output staging (4 x 32 rows x 264 B) reuses the ring
   const int total = p.tiles_m * p.tiles_n;
   const int grid = (total + 7) / 8 * 8;
