@@ -299,30 +299,37 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
         (&sc.w[0][0])[i] = (int)((unsigned)(&sn.w[0][0])[i] >> sh);
       }
     }
+    // first half: the k step 0 products and the LDS reads of the next unit (early, so that their latency
+    // is over long before the end of the step); second half: the k step 1 products, the DMA requests
+    // and the scale reads.  The split also keeps the two products of one accumulator apart.
+    read_unit((J + 2) & 7, fl, LKIND == 1 || LKIND == 2);
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+        acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+            fa.v[mb][0], fw.v[nb][0], acc[AH][WH][mb][nb], 0, 0, 0, sc.a[AH][mb], 0, sc.w[WH][nb]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (J == 0) load_scale_chunk(t);
     load_unit((t + 9) >> 2, std::integral_constant<int, (J + 1) & 3>{}, (J + 1) & 7);
-    read_unit((J + 2) & 7, fl, LKIND == 1 || LKIND == 2);
     if (Q == 3) read_scales((t >> 2) + 1, sn);
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
+      for (int mb = 0; mb < 2; ++mb)
+        acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+            fa.v[mb][1], fw.v[nb][1], acc[AH][WH][mb][nb], 0, 0, 2, sc.a[AH][mb], 2, sc.w[WH][nb]);
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-          if (ks == 0)
-            acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                fa.v[mb][0], fw.v[nb][0], acc[AH][WH][mb][nb], 0, 0, 0, sc.a[AH][mb], 0, sc.w[WH][nb]);
-          else
-            acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                fa.v[mb][1], fw.v[nb][1], acc[AH][WH][mb][nb], 0, 0, 2, sc.a[AH][mb], 2, sc.w[WH][nb]);
-        }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // one LDS read
-      if (Q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // + one scale read
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one matrix instruction
-      if (i & 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);      // one DMA request
-      if (J == 0 && (i == 0 || i == 2)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one matrix instruction
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);                  // one DMA request
+      if (J == 0 && i < 2) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+      if (Q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);      // two scale reads
     }
     // Unit t+3 must have landed (mine: the wait; everybody's: the barrier), and every wave must be done
     // reading the slot of unit t+2 before the next step refills it.  Requested after unit t+3: six
