@@ -308,7 +308,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
         acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            fa.v[mb][0], fw.v[nb][0], acc[AH][WH][mb][nb], 0, 0, 0, sc.a[AH][mb], 0, sc.w[WH][nb]);
+            fw.v[nb][0], fa.v[mb][0], acc[AH][WH][mb][nb], 0, 0, 0, sc.w[WH][nb], 0, sc.a[AH][mb]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
         acc[AH][WH][mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            fa.v[mb][1], fw.v[nb][1], acc[AH][WH][mb][nb], 0, 0, 2, sc.a[AH][mb], 2, sc.w[WH][nb]);
+            fw.v[nb][1], fa.v[mb][1], acc[AH][WH][mb][nb], 0, 0, 2, sc.w[WH][nb], 2, sc.a[AH][mb]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one matrix instruction
@@ -349,59 +349,59 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
     step(t + 7, std::integral_constant<int, 7>{}, fy, fq, fx);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // the trailing (empty) DMA requests
-  __syncthreads();  // the staging below reuses the ring
 
-  // ---- epilogue: bias, SwiGLU, 16-bit, transpose through LDS, coalesced rows -------------------------------------
-  // accumulator [a][w][mb][nb]: row = a*128 + wm*64 + mb*32 + 8*(r/4) + 4*h + r%4,
-  // W row (tile-local) = w*128 + wn*64 + nb*32 + l32.  Output columns of the wave: SwiGLU: f0 + wn*64 + [0,64)
-  // (gate from w = 0, up from w = 1); plain: f0 + w*128 + wn*64 + [0,64) for w = 0, 1.
-  constexpr int kORow = 64 * 2 + 8;                    // padded staging row (bytes): 64 columns
-  MSD_LDS char* ost = smem + wave * 32 * kORow;       // 32 rows per wave at a time
-  float bias_v[2][2];
-#pragma unroll
-  for (int w = 0; w < 2; ++w)
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      const int wrow = (SWIGLU ? w * half : w * 128) + f0 + wn * 64 + nb * 32 + l32;
-      bias_v[w][nb] = (p.bias && wrow < p.Nw) ? p.bias[wrow] : 0.f;
-    }
+  // ---- epilogue: bias, SwiGLU, 16-bit, straight from the accumulators ----------------------------------------------
+  // W rows are the first matrix operand, so accumulator [a][w][mb][nb] register r holds
+  // X row a*128 + wm*64 + mb*32 + l32 and W row (tile-local) w*128 + wn*64 + nb*32 + 8*(r/4) + 4*h + r%4:
+  // four consecutive output columns per register quad, written as one 8-byte store (the two halves of
+  // the wave complete 16 bytes, the four quads and two blocks the 128-byte line).  Output columns of the
+  // wave: SwiGLU: f0 + wn*64 + [0,64) (gate from w = 0, up from w = 1); plain: f0 + w*128 + wn*64 + [0,64).
   T* og = (T*)p.out;
+  auto write_tile = [&](auto bias_c) {
+    constexpr bool BIAS = decltype(bias_c)::value;
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+      for (int mb = 0; mb < 2; ++mb) {
+        const int m = m0 + a * 128 + wm * 64 + mb * 32 + l32;
+        T* orow = og + (long long)m * p.Nout;
 #pragma unroll
-      for (int w = 0; w < (SWIGLU ? 1 : 2); ++w) {
+        for (int w = 0; w < (SWIGLU ? 1 : 2); ++w)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+          for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) {
-            float val;
-            if (SWIGLU) {
-              const float g = acc[a][0][mb][nb][r] + bias_v[0][nb];
-              const float u = acc[a][1][mb][nb][r] + bias_v[1][nb];
-              val = g * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * g)) * u;
-            } else {
-              val = acc[a][w][mb][nb][r] + bias_v[w][nb];
+            for (int j = 0; j < 4; ++j) {
+              const int ncol = wn * 64 + nb * 32 + 8 * j + 4 * h;  // first of the four columns, tile-local
+              const int col = f0 + (SWIGLU ? 0 : w * 128) + ncol;
+              const bool col_ok = col < p.Nout;
+              float v[4];
+              if (SWIGLU) {
+                f32x4_t bg = {0.f, 0.f, 0.f, 0.f}, bu = {0.f, 0.f, 0.f, 0.f};
+                if (BIAS) {  // columns past the end read column 0 (never stored)
+                  bg = *(const f32x4_t*)(p.bias + (col_ok ? col : 0));
+                  bu = *(const f32x4_t*)(p.bias + half + (col_ok ? col : 0));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const float g = acc[a][0][mb][nb][4 * j + e] + bg[e];
+                  const float u = acc[a][1][mb][nb][4 * j + e] + bu[e];
+                  v[e] = g * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * g)) * u;
+                }
+              } else {
+                f32x4_t bv = {0.f, 0.f, 0.f, 0.f};
+                if (BIAS) bv = *(const f32x4_t*)(p.bias + (col_ok ? col : 0));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[a][w][mb][nb][4 * j + e] + bv[e];
+              }
+              if (m < p.M && col_ok) {
+                T t4[4] = {E::from_float(v[0]), E::from_float(v[1]), E::from_float(v[2]), E::from_float(v[3])};
+                *(i32x2_t*)(orow + col) = *(const i32x2_t*)t4;
+              }
             }
-            *(MSD_LDS T*)(ost + row * kORow + (nb * 32 + l32) * 2) = E::from_float(val);
-          }
-        }
-        __builtin_amdgcn_wave_barrier();
-        const int col0 = f0 + (SWIGLU ? 0 : w * 128) + wn * 64;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {  // 32 rows x 8 chunks of 16 bytes
-          const int cidx = i * 64 + lane;
-          const int row = cidx >> 3, c16 = cidx & 7;
-          const int m = m0 + a * 128 + wm * 64 + mb * 32 + row;
-          const int col = col0 + c16 * 8;
-          const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16);
-          const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORow + c16 * 16 + 8);
-          if (m < p.M && col < p.Nout) *(i32x4_t*)(og + (long long)m * p.Nout + col) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
-        }
-        __builtin_amdgcn_wave_barrier();
       }
+  };
+  if (p.bias) write_tile(std::true_type{});
+  else write_tile(std::false_type{});
 #endif
 }
 
