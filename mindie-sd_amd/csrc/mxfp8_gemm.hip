@@ -11,12 +11,12 @@
 // v_mfma_scale_f32_32x32x64_f8f6f4 the lane (row = lane%32, half h = lane/32) holds K-values
 // 16h..16h+15 (registers 0-3) and 32+16h..32+16h+15 (registers 4-7) of the 64-wide step, i.e. two
 // 16-byte chunks, one from each 32-element MX block; the scale byte supplied by lane (row, h) is
-// applied to MX block h of that row.  X is the A operand (row m), W the B operand (column n).
+// applied to MX block h of that row.  W is the first matrix operand (accumulator rows n), X the second
+// (accumulator columns m): a lane then owns four consecutive output columns per register quad.
 //
-// Workgroup tile: 256 rows of X x 256 rows of W (for SwiGLU: 128 gate rows f0.. and the 128 up
-// rows F+f0.., so both halves of an output element meet in the same lane and register), K step
-// 128 bytes, LDS double buffered (2 x 64 KiB) and filled by LDS-DMA; 8 waves as 4 (M) x 2 (N), each
-// 64 x 128 = 2 x 4 MFMA blocks.  LDS rows are 128 bytes; 16-byte chunk c of row r sits at
+// Workgroup tile: 256 rows of X x 256 rows of W (for SwiGLU: 128 gate rows f0.. and the 128 up rows
+// F+f0.., so both halves of an output element meet in the same lane and register); the kernel comment
+// below describes how the tile is walked.  LDS rows are 128 bytes; 16-byte chunk c of row r sits at
 // chunk c ^ ((r >> 1) & 7) (bank-conflict free for the 16-byte operand reads).
 #include "common.hpp"
 

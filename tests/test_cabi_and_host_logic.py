@@ -148,7 +148,10 @@ def test_op_schemas_and_fake_impls():
     out, lse = torch.ops.mindiesd.flash_attention_fwd(q, q, q)
     assert out.shape == q.shape and lse.shape == (2, 4, 300)
     schema = str(torch.ops.mindiesd.block_sparse_attention.default._schema)
-    for piece in ("Tensor? block_sparse_mask=None", "int[] block_shape=[128, 128]", "str q_input_layout=\"BNSD\"",
+    block_shape = [a for a in torch.ops.mindiesd.block_sparse_attention.default._schema.arguments
+                   if a.name == "block_shape"][0]
+    assert block_shape.default_value == [128, 128] and str(block_shape.type) == "List[int]"
+    for piece in ("Tensor? block_sparse_mask=None", "int[] block_shape=", "str q_input_layout=\"BNSD\"",
                   "int num_key_value_heads=1", "float scale_value=1.", "int softmax_lse_flag=0"):
         assert piece in schema, (piece, schema)
 
