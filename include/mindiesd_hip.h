@@ -45,6 +45,31 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
                                  long long o_sb, long long o_sn, long long o_ss,
                                  float scale, hipStream_t stream);
 
+/* Dense attention with the options of the reference's vendor kernels that the entry point above leaves
+ * out:
+ *   seq_meta != NULL: packed variable-length sequences (layout "TND").  q/out are [Tq][N][128], k/v
+ *     [Tk][Nkv][128] (pass batch strides 0); B = number of sequences, Sq / Skv = the longest query / key
+ *     count; seq_meta is a device array int32 [B][4] = {first query token, query count, first key token,
+ *     key count}.  Replaces torch_npu.npu_fusion_attention(input_layout="TND", actual_seq_qlen,
+ *     actual_seq_kvlen) as called by attention_forward_varlen
+ *     (mindiesd/layers/flash_attn/attention_forward_varlen.py:141-149).  lse and mask must be NULL.
+ *   causal != 0: key j is visible to query i iff j <= i + (Skv - Sq), the lower triangle aligned to the
+ *     bottom-right corner (the vendor kernel's sparse_mode = 3, attention_forward_varlen.py:134-136).
+ *   mask != NULL: boolean mask, one byte per (query, key), non-zero = attend, keys contiguous, element
+ *     strides m_sb / m_sn (0 = broadcast over batch / heads) and m_sq.  Replaces the atten_mask argument
+ *     of the fused wrappers (prompt_flash_attn.py:46-52, fused_attn_score.py:46-52; they pass the
+ *     inverted mask, this entry point takes it as the caller of attention_forward gives it).
+ * A query row without any visible key gives zeros (and lse = -inf). */
+int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                         int B, int N, int Nkv, int Sq, int Skv, int D,
+                                         long long q_sb, long long q_sn, long long q_ss,
+                                         long long k_sb, long long k_sn, long long k_ss,
+                                         long long v_sb, long long v_sn, long long v_ss,
+                                         long long o_sb, long long o_sn, long long o_ss,
+                                         float scale, const int* seq_meta, int causal,
+                                         const unsigned char* mask, long long m_sb, long long m_sn, long long m_sq,
+                                         hipStream_t stream);
+
 /* Benchmark hook: selects one of the compiled dense kernel variants (0 = default). */
 void mindiesd_set_dense_variant(int variant);
 

@@ -47,6 +47,12 @@ struct FaParams {
   int QB;
   const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
   int map_mode;      // 0: consecutive query tiles of a head share an XCD; 1: linear block order
+  // general mode (MODE = 1 instantiations only)
+  const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
+                              // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count
+  int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
+  const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
+  long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
 };
 
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
@@ -85,7 +91,7 @@ __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu
 
 // Register budget: 8 wavefronts per CU (two per SIMD) in every configuration, i.e. at most 256
 // registers per lane; the 4-wave configurations run two workgroups per CU.
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -119,6 +125,20 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
   const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
   const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+  // sequence lengths of this (batch) problem; packed sequences bring their own and their token offsets
+  int Sq = p.Sq, Skv = p.Skv;
+  if (MODE && p.seq_meta) {
+    const int* meta = p.seq_meta + 4 * b;
+    Sq = meta[1];
+    Skv = meta[3];
+    if (q0 >= Sq) return;  // the grid is sized for the longest sequence
+    qg += (long long)meta[0] * p.q_ss;
+    og += (long long)meta[0] * p.o_ss;
+    kg += (long long)meta[2] * p.k_ss;
+    vg += (long long)meta[2] * p.v_ss;
+  }
+  const int causal_shift = Skv - Sq;
 
   // ---- tile stream ----------------------------------------------------------------------------
   // Dense: key tiles 0, BN, 2*BN, ...  Sparse: a workgroup owns kBM/128 query blocks (one per group
@@ -134,7 +154,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #pragma unroll
   for (int qb = 0; qb < C::kNQB; ++qb) {
     const int qrow = q0 + wave * QPW + qb * 32 + l32;
-    const bool ok = qrow < p.Sq;
+    const bool ok = qrow < Sq;
     const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * h;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
@@ -174,9 +194,9 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   // is a scalar offset.  Rows past the end of the sequence are out of the buffer's range and read
   // as zeros (their scores are masked to -inf below).
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kg, 0, (int)(((long long)(p.Skv - 1) * p.k_ss + C::kD) * 2), 0x00020000);
+      (void*)kg, 0, Skv > 0 ? (int)(((long long)(Skv - 1) * p.k_ss + C::kD) * 2) : 0, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vg, 0, (int)(((long long)(p.Skv - 1) * p.v_ss + C::kD) * 2), 0x00020000);
+      (void*)vg, 0, Skv > 0 ? (int)(((long long)(Skv - 1) * p.v_ss + C::kD) * 2) : 0, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
   int k_voff[C::kGroupsPerWave], v_voff[C::kGroupsPerWave];
 #pragma unroll
@@ -235,7 +255,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   };
   // cur_*: the tile being computed; nxt_*: the tile being fetched.  key0 < 0 marks the end.
   int cur_key0 = -1, nxt_key0 = -1, cur_fl = 0, nxt_fl = 0, sub = 0;
-  const int dense_tiles = (p.Skv + BN - 1) / BN;
+  // causal: the last row of this workgroup sees keys <= q0 + kBM - 1 + shift; later tiles are skipped
+  int kv_lim = Skv;
+  if (MODE && p.causal) kv_lim = max(0, min(Skv, q0 + C::kBM + causal_shift));
+  const int dense_tiles = (kv_lim + BN - 1) / BN;
+  const unsigned char* mask_g = nullptr;
+  if (MODE && p.mask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
   auto stream_next = [&](int& key0, int& fl) {  // sparse: produce the tile after the one produced last
     if (sub > 0) {  // remaining sub-tiles of the current 128-key block
       key0 = key0 + BN;
@@ -313,17 +338,48 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
 
     // ---- mask keys past the end of the sequence (last tile only) --------------------------------
-    if (key0 + BN > p.Skv) {
+    if (key0 + BN > Skv) {
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-          if (key >= p.Skv) {
+          if (key >= Skv) {
 #pragma unroll
             for (int qb = 0; qb < C::kNQB; ++qb) sacc[kb][qb][r] = -INFINITY;
           }
         }
+    }
+    if (MODE) {
+      // causal: only tiles that reach past the diagonal of this wave's first row need element tests
+      if (p.causal && key0 + BN - 1 > q0 + wave * QPW + causal_shift) {
+#pragma unroll
+        for (int qb = 0; qb < C::kNQB; ++qb) {
+          const int last_visible = q0 + wave * QPW + qb * 32 + l32 + causal_shift;
+#pragma unroll
+          for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+              if (key > last_visible) sacc[kb][qb][r] = -INFINITY;
+            }
+        }
+      }
+      // boolean mask: one byte per (query, key); a lane tests the 16 x kNKB keys of its own query row
+      if (mask_g) {
+#pragma unroll
+        for (int qb = 0; qb < C::kNQB; ++qb) {
+          const int qrow = min(q0 + wave * QPW + qb * 32 + l32, Sq - 1);
+          const unsigned char* mrow = mask_g + (long long)qrow * p.m_sq;
+#pragma unroll
+          for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+              if (key < Skv && mrow[key] == 0) sacc[kb][qb][r] = -INFINITY;
+            }
+        }
+      }
     }
 
     // ---- online softmax in the exp2 domain with a lazily moved reference maximum ------------------
@@ -425,13 +481,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   // Each wave stages only its own rows, and a wave's LDS operations execute in order, so no
   // workgroup barrier is needed here (the loop above ended with one).
   MSD_LDS char* ost = smem + wave * 32 * C::kORowBytes;
-  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
 #pragma unroll
   for (int qb = 0; qb < C::kNQB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int qrow_l = q0 + wave * QPW + qb * 32 + l32;
-    if (p.lse && h == 0 && qrow_l < p.Sq) {
+    if (p.lse && h == 0 && qrow_l < Sq) {
       const long long li = ((long long)b * p.N + n) * p.Sq + qrow_l;
       p.lse[li] = l_tot > 0.f ? m_run[qb] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
     }
@@ -454,7 +509,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       // rows are padded by 8 bytes, so a 16-byte chunk is read as two 8-byte halves
       const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * C::kORowBytes + c16 * 16);
       const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * C::kORowBytes + c16 * 16 + 8);
-      if (qrow < p.Sq) {
+      if (qrow < Sq) {
         i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
         *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = v;
       }
@@ -719,10 +774,10 @@ static int launch_fa_pp(const FaParams& p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
-  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED>;
+  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE>;
   // per device and idempotent, so it is simply repeated on every launch
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
     return MSD_ERR_LAUNCH;
@@ -826,6 +881,29 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
     }
   }
   return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1>(p, stream);
+}
+
+// Dense attention with the options the plain entry point leaves out: packed variable-length sequences,
+// a causal mask aligned to the bottom-right corner, a boolean attention mask.  Rows whose keys are all
+// masked give zeros.
+int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                         int B, int N, int Nkv, int Sq, int Skv, int D, long long q_sb, long long q_sn,
+                                         long long q_ss, long long k_sb, long long k_sn, long long k_ss,
+                                         long long v_sb, long long v_sn, long long v_ss, long long o_sb,
+                                         long long o_sn, long long o_ss, float scale, const int* seq_meta, int causal,
+                                         const unsigned char* mask, long long m_sb, long long m_sn, long long m_sq,
+                                         hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (seq_meta && (mask || lse)) return MSD_ERR_UNSUPPORTED;  // packed sequences: neither mask nor lse layout defined
+  if (mask && (m_sb < 0 || m_sn < 0 || m_sq < Skv)) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  p.map_mode = g_map_mode;
+  p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
+  p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1, 1>(p, stream);
 }
 
 }  // extern "C"

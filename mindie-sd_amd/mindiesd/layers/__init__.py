@@ -1,4 +1,4 @@
 from . import _custom_ops  # noqa: F401  (declares torch.ops.mindiesd.*)
-from .flash_attn import attention_forward, sparse_attention
+from .flash_attn import attention_forward, attention_forward_varlen, sparse_attention
 
-__all__ = ["attention_forward", "sparse_attention"]
+__all__ = ["attention_forward", "attention_forward_varlen", "sparse_attention"]

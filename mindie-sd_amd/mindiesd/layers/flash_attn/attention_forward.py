@@ -16,7 +16,7 @@ def attention_forward(query, key, value, attn_mask=None, scale=None, fused=True,
     The output has the layout and dtype of ``query``.
 
     Args:
-        attn_mask: boolean [Sq, Skv] or [B, N, Sq, Skv], True = attend (unfused path only).
+        attn_mask: [Sq, Skv] or [B|1, N|1, Sq, Skv], True / non-zero = attend.
         scale: float softmax scale, default head_dim ** -0.5.
         fused: True runs the HIP flash-attention kernel, False the unfused torch math.
         kwargs: ``opt_mode`` in {'runtime' (default), 'static', 'manual'}; with 'manual',

@@ -24,39 +24,105 @@ def _strides_bns(t, layout):
     return t.stride(0), t.stride(2), t.stride(1)
 
 
-def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False):
-    """softmax(scale * Q K^T) V on the GPU.  ``layout`` is 'BNSD' or 'BSND'; the output has the
-    input's layout and dtype.  Grouped-query attention is supported (N % N_kv == 0)."""
+def _check_qkv(query, key, value):
     for name, t in (("query", query), ("key", key), ("value", value)):
         if not t.is_cuda:
             raise ParametersInvalid(f"The fused attention kernel needs GPU tensors, but {name} is on {t.device}.")
     if query.dtype not in _native.DTYPE_CODE or key.dtype != query.dtype or value.dtype != query.dtype:
         raise ParametersInvalid(f"The fused attention kernel supports bf16/fp16 with equal q/k/v dtypes, "
                                 f"but got {query.dtype}, {key.dtype}, {value.dtype}.")
+    d = query.shape[-1]
+    if d != HEAD_DIM or key.shape[-1] != d or value.shape[-1] != d:
+        raise ParametersInvalid(f"The fused attention kernel supports head_dim == {HEAD_DIM}, but got {d}.")
+
+
+def _aligned(t):
+    return t if (t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1])
+                 and t.data_ptr() % 16 == 0) else t.contiguous()
+
+
+def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, attn_mask=None, causal=False):
+    """softmax(scale * Q K^T) V on the GPU.  ``layout`` is 'BNSD' or 'BSND'; the output has the
+    input's layout and dtype.  Grouped-query attention is supported (N % N_kv == 0).
+
+    ``attn_mask``: [Sq, Skv] or [B|1, N|1, Sq, Skv], non-zero / True = attend (the reference's fused
+    wrappers hand the vendor kernel ``~mask.to(torch.bool)``, prompt_flash_attn.py:46-47); ``causal``
+    keeps key j for query i iff j <= i + (Skv - Sq).  Rows without any visible key give zeros."""
+    _check_qkv(query, key, value)
     if layout == "BNSD":
         b, n, sq, d = query.shape
         nkv, skv = key.shape[1], key.shape[2]
     else:
         b, sq, n, d = query.shape
         skv, nkv = key.shape[1], key.shape[2]
-    if d != HEAD_DIM or key.shape[-1] != d or value.shape[-1] != d:
-        raise ParametersInvalid(f"The fused attention kernel supports head_dim == {HEAD_DIM}, but got {d}.")
     if key.shape != value.shape or key.shape[0] != b or n % nkv != 0:
         raise ParametersInvalid("Inconsistent query/key/value shapes.")
-    fix = lambda t: t if (t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1])
-                          and t.data_ptr() % 16 == 0) else t.contiguous()
-    query, key, value = fix(query), fix(key), fix(value)
+    query, key, value = _aligned(query), _aligned(key), _aligned(value)
     out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
     lse = torch.empty((b, n, sq), dtype=torch.float32, device=query.device) if return_lse else None
+    strides = (*_strides_bns(query, layout), *_strides_bns(key, layout), *_strides_bns(value, layout),
+               *_strides_bns(out, layout))
     with torch.cuda.device(query.device):
-        rc = _native.lib().mindiesd_flash_attention_fwd(
-            query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
-            lse.data_ptr() if lse is not None else None, _native.DTYPE_CODE[query.dtype],
-            b, n, nkv, sq, skv, d,
-            *_strides_bns(query, layout), *_strides_bns(key, layout), *_strides_bns(value, layout),
-            *_strides_bns(out, layout), float(scale), _native.stream_ptr(query.device))
-    _native.check(rc, "mindiesd_flash_attention_fwd")
+        if attn_mask is None and not causal:
+            rc = _native.lib().mindiesd_flash_attention_fwd(
+                query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
+                lse.data_ptr() if lse is not None else None, _native.DTYPE_CODE[query.dtype],
+                b, n, nkv, sq, skv, d, *strides, float(scale), _native.stream_ptr(query.device))
+            _native.check(rc, "mindiesd_flash_attention_fwd")
+        else:
+            mask, m_sb, m_sn, m_sq = None, 0, 0, 0
+            if attn_mask is not None:
+                mask = attn_mask
+                if mask.dim() == 2:
+                    mask = mask[None, None]
+                if (mask.dim() != 4 or mask.shape[-2:] != (sq, skv) or mask.shape[0] not in (1, b)
+                        or mask.shape[1] not in (1, n)):
+                    raise ParametersInvalid(f"attn_mask must be [Sq, Skv] or [B|1, N|1, Sq, Skv] = [{b}|1, {n}|1, {sq}, {skv}], "
+                                            f"but got {tuple(attn_mask.shape)}.")
+                mask = mask.to(device=query.device, dtype=torch.bool)
+                if mask.stride(-1) != 1:
+                    mask = mask.contiguous()
+                m_sb = mask.stride(0) if mask.shape[0] > 1 else 0
+                m_sn = mask.stride(1) if mask.shape[1] > 1 else 0
+                m_sq = mask.stride(2) if sq > 1 else skv
+            rc = _native.lib().mindiesd_flash_attention_general_fwd(
+                query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
+                lse.data_ptr() if lse is not None else None, _native.DTYPE_CODE[query.dtype],
+                b, n, nkv, sq, skv, d, *strides, float(scale), None, int(bool(causal)),
+                mask.data_ptr() if mask is not None else None, m_sb, m_sn, m_sq, _native.stream_ptr(query.device))
+            _native.check(rc, "mindiesd_flash_attention_general_fwd")
     return (out, lse) if return_lse else out
+
+
+def flash_attention_varlen(q, k, v, seqlens_q, seqlens_k, scale, causal=False):
+    """Packed sequences: q [Tq, N, D], k / v [Tk, Nkv, D]; sequence i owns ``seqlens_q[i]`` query tokens and
+    ``seqlens_k[i]`` key tokens, stored back to back.  Returns [Tq, N, D]."""
+    _check_qkv(q, k, v)
+    if q.dim() != 3 or k.shape != v.shape or k.dim() != 3 or q.shape[1] % k.shape[1] != 0:
+        raise ParametersInvalid("Inconsistent query/key/value shapes.")
+    if len(seqlens_q) != len(seqlens_k) or len(seqlens_q) == 0:
+        raise ParametersInvalid("cu_seqlens_q and cu_seqlens_k must describe the same, non-zero number of sequences.")
+    if min(seqlens_q) < 0 or min(seqlens_k) < 0 or sum(seqlens_q) != q.shape[0] or sum(seqlens_k) != k.shape[0]:
+        raise ParametersInvalid("The cumulative sequence lengths do not match the token dimensions of q / k.")
+    q, k, v = _aligned(q), _aligned(k), _aligned(v)
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    meta, oq, ok = [], 0, 0
+    for lq, lk in zip(seqlens_q, seqlens_k):
+        meta += [oq, lq, ok, lk]
+        oq += lq
+        ok += lk
+    if max(seqlens_q) == 0:
+        return out
+    meta_t = torch.tensor(meta, dtype=torch.int32).to(q.device, non_blocking=True)
+    tn = lambda t: (0, t.stride(1), t.stride(0))  # (batch, head, token) strides of a [T, N, D] tensor
+    with torch.cuda.device(q.device):
+        rc = _native.lib().mindiesd_flash_attention_general_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None, _native.DTYPE_CODE[q.dtype],
+            len(seqlens_q), q.shape[1], k.shape[1], max(seqlens_q), max(max(seqlens_k), 1), q.shape[2],
+            *tn(q), *tn(k), *tn(v), *tn(out), float(scale), meta_t.data_ptr(), int(bool(causal)), None, 0, 0, 0,
+            _native.stream_ptr(q.device))
+    _native.check(rc, "mindiesd_flash_attention_general_fwd")
+    return out
 
 
 @register_op_mi355x("hip_flash_attn", "prompt_flash_attn", "fused_attn_score", "ascend_laser_attention")
@@ -72,12 +138,9 @@ class HipFlashAttention(AttentionOperateBase):
 
     @classmethod
     def _run(cls, attn_param, query, key, value, mask, scale):
-        if mask is not None:
-            raise ParametersInvalid("attn_mask is not supported by the fused HIP kernel; "
-                                    "call attention_forward(..., fused=False) for masked attention.")
         if scale is None:
             scale = attn_param.head_dim ** -0.5
-        return flash_attention(query, key, value, scale, "BNSD" if attn_param.head_first else "BSND")
+        return flash_attention(query, key, value, scale, "BNSD" if attn_param.head_first else "BSND", attn_mask=mask)
 
     # The kernel is stride-generic, so the three "layouts" of the reference differ only in how the
     # caller's tensors are viewed: nothing is transposed or copied for any of them.

@@ -60,6 +60,38 @@ def attention_math_rows(query, key, value, scale=None, row_chunk=4096, q_rows=No
     return torch.cat(outs, dim=2)
 
 
+def causal_keep_mask(sq, skv):
+    """Boolean [sq, skv] mask of the vendor kernel's ``sparse_mode=3`` ("rightDownCausal", the mode
+    attention_forward_varlen.py:134-136 selects): the lower triangle aligned to the bottom-right
+    corner, i.e. key j is visible to query i iff j <= i + (skv - sq)."""
+    i = torch.arange(sq)[:, None]
+    j = torch.arange(skv)[None, :]
+    return j <= i + (skv - sq)
+
+
+def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale=None, causal=False):
+    """Packed [T, N, D] sequences (attention_forward_varlen.py:59-149): every sequence is an independent
+    ``attention_math`` problem over its own slice of q and k / v (grouped-query heads repeated), with the
+    bottom-right aligned causal mask when ``causal``.  Rows without a visible key (possible when a
+    sequence has fewer keys than queries) are defined as zeros here."""
+    t, n, d = q.shape
+    nkv = k.shape[1]
+    out = torch.zeros(q.shape, dtype=q.dtype)
+    for i in range(len(cu_seqlens_q) - 1):
+        q0, q1, k0, k1 = int(cu_seqlens_q[i]), int(cu_seqlens_q[i + 1]), int(cu_seqlens_k[i]), int(cu_seqlens_k[i + 1])
+        if q1 == q0 or k1 == k0:
+            continue
+        qs = q[q0:q1].transpose(0, 1)[None]
+        ks = k[k0:k1].transpose(0, 1).repeat_interleave(n // nkv, dim=0)[None]
+        vs = v[k0:k1].transpose(0, 1).repeat_interleave(n // nkv, dim=0)[None]
+        mask = causal_keep_mask(q1 - q0, k1 - k0) if causal else None
+        o = attention_math(qs, ks, vs, mask, scale, head_first=True)
+        if mask is not None:
+            o = torch.where(mask.any(dim=-1)[None, None, :, None], o, torch.zeros((), dtype=o.dtype))
+        out[q0:q1] = o[0].transpose(0, 1)
+    return out
+
+
 def attention_fp64(query, key, value, scale, keep=None):
     """Brute-force fp64 softmax(scale QK^T)V for one [S,D] problem; pins attention_math."""
     q = query.double().numpy()

@@ -1,0 +1,117 @@
+"""GPU parity of the general mode of the flash-attention kernel (boolean attention mask, bottom-right aligned
+causal mask, packed variable-length sequences) vs the CPU oracle; bf16 tolerance as for the dense kernel:
+max-abs <= 2e-2 and cosine >= 0.9999."""
+import pytest
+import torch
+
+from oracle.attention import attention_math, attention_varlen, causal_keep_mask, cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(shape, seed, dtype=torch.bfloat16, mul=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * mul).to(dtype)
+
+
+def _check(out, ref, max_abs=2e-2, min_cos=0.9999):
+    assert not torch.isnan(out.float()).any()
+    err = (out.float() - ref.float()).abs().max().item()
+    assert err <= max_abs, f"max-abs {err}"
+    assert cosine(out, ref) >= min_cos, f"cosine {cosine(out, ref)}"
+
+
+@pytest.mark.parametrize("head_first", [True, False])
+@pytest.mark.parametrize("mask_shape", ["2d", "b1", "bn"])
+def test_fused_attention_with_boolean_mask(cuda, mask_shape, head_first):
+    import mindiesd
+    b, n, sq, skv = 2, 3, 300, 421
+    q = _rand((b, n, sq, 128), 1)
+    k = _rand((b, n, skv, 128), 2)
+    v = _rand((b, n, skv, 128), 3)
+    g = torch.Generator().manual_seed(4)
+    shape = {"2d": (sq, skv), "b1": (b, 1, sq, skv), "bn": (b, n, sq, skv)}[mask_shape]
+    mask = torch.rand(shape, generator=g) > 0.4
+    mask[..., 5] = True  # every row keeps at least one key
+    full = mask if mask.dim() == 4 else mask[None, None]
+    ref = attention_math(q, k, v, full.expand(b, n, sq, skv), head_first=True)
+    args = (q, k, v) if head_first else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = mindiesd.attention_forward(*(t.to(cuda) for t in args), attn_mask=mask.to(cuda), head_first=head_first).cpu()
+    _check(out if head_first else out.transpose(1, 2), ref)
+
+
+def test_mask_dtypes_and_fully_masked_rows(cuda):
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    q, k, v = _rand((1, 2, 130, 128), 5), _rand((1, 2, 200, 128), 6), _rand((1, 2, 200, 128), 7)
+    mask = torch.zeros(130, 200, dtype=torch.int32)
+    mask[:, 17] = 3          # non-zero = attend
+    mask[7] = 0              # a row without any visible key
+    out = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", attn_mask=mask.to(cuda)).cpu()
+    assert not out[:, :, 7].any()
+    rows = [r for r in range(130) if r != 7]
+    assert torch.equal(out[:, :, rows], v[:, :, 17:18].expand(1, 2, 129, 128))  # one visible key: the output is its value row
+
+
+@pytest.mark.parametrize("sq,skv", [(256, 256), (300, 300), (77, 500), (500, 77), (1000, 1300)])
+def test_causal_bottom_right(cuda, sq, skv):
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    q, k, v = _rand((1, 4, sq, 128), 8), _rand((1, 2, skv, 128), 9), _rand((1, 2, skv, 128), 10)
+    out, lse = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", return_lse=True, causal=True)
+    keep = causal_keep_mask(sq, skv)
+    kk, vv = k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1)
+    ref = attention_math(q, kk, vv, keep, head_first=True)
+    seen = keep.any(-1)
+    ref = torch.where(seen[None, None, :, None], ref, torch.zeros((), dtype=ref.dtype))
+    _check(out.cpu(), ref)
+    assert not out.cpu()[:, :, ~seen].any()
+    s = (q.float() @ kk.float().transpose(-1, -2)) * 128 ** -0.5
+    want_lse = torch.logsumexp(s.masked_fill(~keep, float("-inf")), dim=-1)
+    assert torch.allclose(lse.cpu()[:, :, seen], want_lse[:, :, seen], atol=5e-3, rtol=0)
+    assert torch.isinf(lse.cpu()[:, :, ~seen]).all()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_forward_varlen(cuda, causal):
+    import mindiesd
+    lens_q, lens_k = [300, 1, 0, 513, 40], [300, 77, 5, 256, 900]
+    cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+    cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+    q, k, v = _rand((sum(lens_q), 4, 128), 11), _rand((sum(lens_k), 2, 128), 12), _rand((sum(lens_k), 2, 128), 13)
+    out = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu_q.to(cuda), cu_k.to(cuda),
+                                            causal=causal).cpu()
+    ref = attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal)
+    assert out.shape == q.shape and out.dtype == q.dtype
+    _check(out, ref)
+    # lists of python ints work as well, and a custom scale
+    out2 = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu_q.tolist(), cu_k.tolist(),
+                                             softmax_scale=0.05, causal=causal).cpu()
+    _check(out2, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), scale=0.05, causal=causal))
+
+
+def test_varlen_single_sequence_equals_dense(cuda):
+    import mindiesd
+    q, k, v = _rand((700, 2, 128), 14, mul=0.5), _rand((700, 2, 128), 15, mul=0.5), _rand((700, 2, 128), 16, mul=0.5)
+    a = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), [0, 700], [0, 700])
+    b = mindiesd.attention_forward(q[None].to(cuda), k[None].to(cuda), v[None].to(cuda))
+    assert torch.equal(a, b[0])
+
+
+def test_varlen_and_mask_errors(cuda):
+    import mindiesd
+    from mindiesd import ParametersInvalid
+    q = torch.randn(10, 2, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(ParametersInvalid, match="Unsupported parameters in varlen attention"):
+        mindiesd.attention_forward_varlen(q, q, q, [0, 10], [0, 10], window_size=3)
+    with pytest.raises(ParametersInvalid, match="dropout_p"):
+        mindiesd.attention_forward_varlen(q, q, q, [0, 10], [0, 10], dropout_p=0.1)
+    with pytest.raises(ParametersInvalid, match="3D"):
+        mindiesd.attention_forward_varlen(q[None], q[None], q[None], [0, 10], [0, 10])
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward_varlen(q, q, q, [0, 9], [0, 10])
+    with pytest.raises(ParametersInvalid):
+        mindiesd.attention_forward_varlen(q, q, q, [0, 4, 10], [0, 10])
+    x = torch.randn(1, 64, 2, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(ParametersInvalid, match="attn_mask"):
+        mindiesd.attention_forward(x, x, x, attn_mask=torch.ones(3, 64, 64, dtype=torch.bool, device=cuda))
+    with pytest.raises(ParametersInvalid, match="attn_mask"):
+        mindiesd.attention_forward(x, x, x, attn_mask=torch.ones(63, 64, dtype=torch.bool, device=cuda))

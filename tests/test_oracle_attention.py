@@ -123,3 +123,44 @@ def test_tolerance_rules():
     assert ref_compare(g, g + torch.tensor([0.005, 0.02, 0.02]), 2 ** -6)[1]
     assert not ref_compare(g, g + torch.tensor([0.02, 0.0, 0.0]), 2 ** -6)[1]
     assert data_compare(g + 1e-4, g) and not data_compare(g + 0.2, g)
+
+
+# ---- causal mask (bottom-right aligned) and packed variable-length sequences ---------------------------------
+def test_causal_keep_mask_closed_forms():
+    from oracle.attention import causal_keep_mask
+    # square: the ordinary lower triangle
+    assert torch.equal(causal_keep_mask(5, 5), torch.ones(5, 5).tril().bool())
+    # more keys than queries: the last query sees everything, the first sees skv - sq + 1 keys
+    m = causal_keep_mask(3, 7)
+    assert torch.equal(m, torch.ones(3, 7).tril(diagonal=4).bool()) and m[-1].all() and int(m[0].sum()) == 5
+    # fewer keys than queries: the first sq - skv queries see nothing, the last sees all keys
+    m = causal_keep_mask(6, 2)
+    assert not m[:4].any() and m[-1].all() and torch.equal(m, torch.ones(6, 2).tril(diagonal=-4).bool())
+
+
+def test_attention_varlen_matches_sdpa_per_sequence():
+    from oracle.attention import attention_varlen, causal_keep_mask
+    g = torch.Generator().manual_seed(3)
+    lens_q, lens_k = [5, 0, 17, 9], [5, 4, 30, 3]
+    cu_q = [0] + list(torch.tensor(lens_q).cumsum(0))
+    cu_k = [0] + list(torch.tensor(lens_k).cumsum(0))
+    q = torch.randn(sum(lens_q), 4, 16, generator=g)
+    k = torch.randn(sum(lens_k), 2, 16, generator=g)
+    v = torch.randn(sum(lens_k), 2, 16, generator=g)
+    for causal in (False, True):
+        got = attention_varlen(q, k, v, cu_q, cu_k, causal=causal)
+        for i, (lq, lk) in enumerate(zip(lens_q, lens_k)):
+            if lq == 0:
+                continue
+            qs = q[cu_q[i]:cu_q[i + 1]].transpose(0, 1)
+            ks = k[cu_k[i]:cu_k[i + 1]].transpose(0, 1).repeat_interleave(2, dim=0)
+            vs = v[cu_k[i]:cu_k[i + 1]].transpose(0, 1).repeat_interleave(2, dim=0)
+            keep = causal_keep_mask(lq, lk) if causal else torch.ones(lq, lk, dtype=torch.bool)
+            want = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=keep)
+            want = torch.where(keep.any(-1)[None, :, None], want, torch.zeros(()))  # SDPA gives NaN for empty rows
+            assert torch.allclose(got[cu_q[i]:cu_q[i + 1]].transpose(0, 1), want, atol=2e-6, rtol=1e-5)
+    # square causal == torch's own is_causal
+    qs = torch.randn(1, 2, 9, 16, generator=g)
+    want = torch.nn.functional.scaled_dot_product_attention(qs, qs, qs, is_causal=True)
+    got = attention_varlen(qs[0].transpose(0, 1), qs[0].transpose(0, 1), qs[0].transpose(0, 1), [0, 9], [0, 9], causal=True)
+    assert torch.allclose(got.transpose(0, 1), want[0], atol=2e-6, rtol=1e-5)
