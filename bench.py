@@ -154,6 +154,28 @@ def extra_dense_1p3b(device, steps, warmup):
             "frac_of_bf16_peak": attn_flops(CFG_1P3B) / m / 1e9 / PEAK_BF16_TFLOPS}
 
 
+def extra_causal_varlen(device, steps, warmup):
+    """General mode of the dense kernel at the 1.3B shape: bottom-right causal mask (about half of the
+    score matrix is skipped) and the same tokens packed as 7 sequences of unequal length."""
+    import torch
+    import mindiesd
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    cfg = CFG_1P3B
+    q, k, v = dense_inputs(cfg, device, seed=2)
+    s, n, d = cfg["S"], cfg["N"], cfg["D"]
+    c_ms, _ = time_steps(lambda: flash_attention(q, k, v, d ** -0.5, "BNSD", causal=True), steps, warmup)
+    lens = [8192, 4096, 300, 12000, 1, 5000, s - 29589]
+    cu = torch.tensor([0] + lens).cumsum(0).tolist()
+    qt, kt, vt = (t[0].transpose(0, 1).contiguous() for t in (q, k, v))
+    v_ms, _ = time_steps(lambda: mindiesd.attention_forward_varlen(qt, kt, vt, cu, cu), steps, warmup)
+    cm, vm = median(c_ms), median(v_ms)
+    causal_flops = 4.0 * n * d * (s * (s + 1) / 2)
+    varlen_flops = 4.0 * n * d * sum(l * l for l in lens)
+    return {"workload": "bf16 B1 N12 S32760 D128: causal; and packed as 7 sequences " + str(lens),
+            "causal_ms": cm, "causal_tflops_unmasked_work": causal_flops / cm / 1e9,
+            "varlen_ms": vm, "varlen_tflops": varlen_flops / vm / 1e9}
+
+
 def extra_sparse(device, steps, warmup, dense_ms):
     """RainFusion block-sparse attention at the 14B 720p shape: top 25 % of key blocks per query
     block + first-frame blocks + diagonal.  Reported with the whole pipeline (permute + pool + mask +
@@ -236,7 +258,7 @@ def extra_fp8(device, steps, warmup):
             "fp8_kernel_speedup_vs_bf16": bm / km,
             "quant_pass_ms": qm, "quant_pass_gbs": quant_bytes / qm / 1e6,
             "fp8_end_to_end_ms": em, "fp8_end_to_end_speedup_vs_bf16": bm / em,
-            "cosine_fp8_vs_bf16_kernel": cos}
+            "cosine_fp8_vs_unquantised_bf16_kernel": cos}
 
 
 def extra_gemm(device, steps, warmup):
@@ -270,7 +292,7 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference kernel for scaling rocprof byte counters)")
     ap.add_argument("--extras-only", default="",
-                    help="comma separated subset of extras to run (dense_wan1p3b,sparse_rf_v3,fp8_attention,"
+                    help="comma separated subset of extras to run (dense_wan1p3b,causal_varlen,sparse_rf_v3,fp8_attention,"
                          "mxfp8_gemm_swiglu)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -323,6 +345,7 @@ def main():
     if not args.no_extras:
         extras = {}
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
+                         ("causal_varlen", lambda: extra_causal_varlen(device, args.steps, args.warmup)),
                          ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
                          ("fp8_attention", lambda: extra_fp8(device, args.steps, args.warmup)),
                          ("mxfp8_gemm_swiglu", lambda: extra_gemm(device, args.steps, args.warmup))):

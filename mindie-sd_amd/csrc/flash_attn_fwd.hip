@@ -116,7 +116,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   if (SPARSE && p.order) work = p.order[blockIdx.x < total ? blockIdx.x : 0];
   if (SPARSE && p.order && blockIdx.x >= total) return;
   const int bn = work / q_tiles;
-  const int qt = work - bn * q_tiles;
+  int qt = work - bn * q_tiles;
+  if (MODE && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
   const int b = bn / p.N;
   const int n = bn - b * p.N;
   const int nkv = n / (p.N / p.Nkv);
@@ -902,8 +903,8 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   p.map_mode = g_map_mode;
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
-  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1, 1>(p, stream);
-  return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1, 1>(p, stream);
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
 }
 
 }  // extern "C"

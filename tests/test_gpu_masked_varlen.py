@@ -93,7 +93,8 @@ def test_varlen_single_sequence_equals_dense(cuda):
     q, k, v = _rand((700, 2, 128), 14, mul=0.5), _rand((700, 2, 128), 15, mul=0.5), _rand((700, 2, 128), 16, mul=0.5)
     a = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), [0, 700], [0, 700])
     b = mindiesd.attention_forward(q[None].to(cuda), k[None].to(cuda), v[None].to(cuda))
-    assert torch.equal(a, b[0])
+    # different tile shapes behind the two entry points: equal up to the summation order
+    assert (a.float() - b[0].float()).abs().max() <= 2.0 ** -8 and cosine(a, b[0]) >= 0.99999
 
 
 def test_varlen_and_mask_errors(cuda):
