@@ -247,6 +247,19 @@ def extra_fp8(device, steps, warmup):
     out8 = f8.fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale)
     out16 = mindiesd.attention_forward(q, k, v, head_first=True)
     cos = float(torch.nn.functional.cosine_similarity(out8.float().flatten(), out16.float().flatten(), dim=0))
+    # the FP8RotateQuantFA recipe: an orthogonal (Hadamard) rotation of q and k spreads the outliers over the
+    # channels before quantisation; here it runs inside the quantisation pass
+    from mindiesd.layers.quant.block_quant import _rot_block_quant
+    had = torch.ones((1, 1), device=device)
+    while had.shape[0] < cfg["D"]:
+        had = torch.cat([torch.cat([had, had], 1), torch.cat([had, -had], 1)], 0)
+    rot = (had / had.shape[0] ** 0.5).to(torch.bfloat16)
+    rot_ms, _ = time_steps(lambda: f8.fp8_attention_forward(q, k, v, q_rot=rot, k_rot=rot), steps, warmup)
+    rq_ms, _ = time_steps(lambda: (_rot_block_quant(q, rot, "BNSD"), _rot_block_quant(k, rot, "BNSD")), steps, warmup)
+    mm_ms, _ = time_steps(lambda: (_block_quant(torch.matmul(q, rot), 128, "BNSD"),
+                                   _block_quant(torch.matmul(k, rot), 128, "BNSD")), steps, warmup)
+    out8r = f8.fp8_attention_forward(q, k, v, q_rot=rot, k_rot=rot)
+    cos_rot = float(torch.nn.functional.cosine_similarity(out8r.float().flatten(), out16.float().flatten(), dim=0))
     f = attn_flops(cfg)
     bm, km, qm, em = median(bf16_ms), median(kern_ms), median(quant_ms), median(e2e_ms)
     # quantisation pass: read q, k once and v twice (maximum, then quantise), write one byte per element
@@ -258,7 +271,10 @@ def extra_fp8(device, steps, warmup):
             "fp8_kernel_speedup_vs_bf16": bm / km,
             "quant_pass_ms": qm, "quant_pass_gbs": quant_bytes / qm / 1e6,
             "fp8_end_to_end_ms": em, "fp8_end_to_end_speedup_vs_bf16": bm / em,
-            "cosine_fp8_vs_unquantised_bf16_kernel": cos}
+            "cosine_fp8_vs_unquantised_bf16_kernel": cos,
+            "rotated_end_to_end_ms": median(rot_ms), "rotated_end_to_end_speedup_vs_bf16": bm / median(rot_ms),
+            "rotate_quant_qk_fused_ms": median(rq_ms), "rotate_quant_qk_matmul_then_quant_ms": median(mm_ms),
+            "cosine_rotated_fp8_vs_unquantised_bf16_kernel": cos_rot}
 
 
 def extra_gemm(device, steps, warmup):

@@ -134,6 +134,13 @@ int mindiesd_lpt_order(const int* blk_cnt, int* order, int total, int max_cnt, h
 int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int B, int N, int S, int D,
                             long long x_sb, long long x_sn, long long x_ss, int block_size, hipStream_t stream);
 
+/* Rotation fused into the quantisation pass: y = x @ rot ([128][128], passed transposed as rot_t, same
+ * 16-bit type as x), y rounded to the 16-bit type, then quantised as above with block_size 128.  Replaces
+ * torch.matmul(query, self.q_rot) / torch.matmul(key, self.k_rot) followed by fa_block_quant_preprocess in
+ * FP8RotateQuantFA.forward (mindiesd/quantization/layer.py:283-296). */
+int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float* scale, int dtype, int B, int N, int S,
+                                int D, long long x_sb, long long x_sn, long long x_ss, hipStream_t stream);
+
 /* V for the FP8 kernel: per-(batch, head, channel) scale = amax/448 over the sequence, codes written
  * transposed ([B][N][128][S rounded up to 128], zero padded, keys permuted inside groups of 64 into
  * the order the matrix instruction consumes).  workspace: mindiesd_fp8_v_quant_workspace_size bytes. */

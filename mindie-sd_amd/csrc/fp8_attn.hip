@@ -96,6 +96,86 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsign
 #endif
 }
 
+// ---- rotation + block quantisation in one pass ------------------------------------------------------------------
+// y = x @ R (R a fixed [128][128] matrix, e.g. a Hadamard rotation that spreads outliers over the channels),
+// y rounded to the 16-bit input type as a separate matmul would leave it, then quantised like
+// block_quant_kernel with 128-token blocks.  x is read once and only the E4M3 codes are written: 3 bytes
+// per element instead of the 7 of matmul + quantisation.
+// One workgroup = one 128-token block; R^T sits in LDS (16-byte chunk c of row n at chunk c ^ (n & 15)); wave w
+// owns tokens 32w..32w+31.  R^T is the first matrix operand, so a lane holds one token and, per register
+// quad, four consecutive output channels = one dword of codes.
+template <int DT>
+__global__ __launch_bounds__(256) void rot_block_quant_kernel(const void* x_, const void* rot_t_, unsigned char* q,
+                                                              float* scale, long long sb, long long sn, long long ss,
+                                                              int N, int S) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using E = Elem<DT>;
+  using T = typename E::type;
+  using X8 = typename E::x8;
+  __shared__ __attribute__((aligned(16))) char rt_lds[128 * 256];
+  __shared__ float red[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, h = lane >> 5;
+  const int blk = blockIdx.x, bn = blockIdx.y;
+  const int b = bn / N, n = bn - b * N;
+  const int nblk = gridDim.x;
+  const T* x = (const T*)x_ + b * sb + n * sn;
+  const int row0 = blk * 128;
+  // R^T [out channel][in channel] -> LDS
+  const char* rt = (const char*)rot_t_;
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int row = pass * 16 + (tid >> 4), c = tid & 15;
+    *(i32x4_t*)(rt_lds + row * 256 + ((c ^ (row & 15)) << 4)) = *(const i32x4_t*)(rt + row * 256 + c * 16);
+  }
+  // this lane's token: in channels 16ks + 8h .. +7 for ks = 0..7
+  const int tok = row0 + wave * 32 + l32;
+  const bool ok = tok < S;
+  X8 xf[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    xf[ks] = *(const X8*)(x + (long long)(ok ? tok : 0) * ss + 16 * ks + 8 * h);
+    if (!ok) xf[ks] = X8{0};
+  }
+  __syncthreads();
+  f32x16_t acc[4];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+    const int row = nb * 32 + l32;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const X8 rf = *(const X8*)(rt_lds + row * 256 + (((2 * ks + h) ^ (row & 15)) << 4));
+      acc[nb] = E::mfma32(rf, xf[ks], acc[nb]);
+    }
+  }
+  // round to the 16-bit type (what a separate matmul would have stored), block maximum
+  float amax = 0.f;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc[nb][r] = (float)E::from_float(acc[nb][r]);
+      amax = fmaxf(amax, fabsf(acc[nb][r]));
+    }
+  amax = block_max_256(amax, red);
+  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  if (tid == 0) scale[(long long)bn * nblk + blk] = sc;
+  if (ok) {
+    unsigned char* qo = q + ((long long)bn * S + tok) * 128;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int w = pack4_e4m3(__fdiv_rn(acc[nb][4 * g], sc), __fdiv_rn(acc[nb][4 * g + 1], sc),
+                                 __fdiv_rn(acc[nb][4 * g + 2], sc), __fdiv_rn(acc[nb][4 * g + 3], sc));
+        *(int*)(qo + nb * 32 + 8 * g + 4 * h) = w;
+      }
+  }
+#endif
+}
+
 // ---- V: per-channel maximum over the sequence ------------------------------------------------------------
 __global__ void fill_u32_kernel(unsigned* p, unsigned v, long long n) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -440,6 +520,25 @@ int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int
   else
     hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
                        x_sn, x_ss, N, S, block_size);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+// y = x @ rot (rot_t = rot transposed, [128][128] contiguous, same 16-bit type as x), rounded to the
+// 16-bit type, then quantised per (head, 128 tokens): codes [B][N][S][128], scale [B][N][ceil(S/128)].
+int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float* scale, int dtype, int B, int N, int S,
+                                int D, long long x_sb, long long x_sn, long long x_ss, hipStream_t stream) {
+  if (!x || !rot_t || !q || !scale || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if ((((uintptr_t)x | (uintptr_t)rot_t) & 15) || ((uintptr_t)q & 3) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
+  const dim3 grid((S + 127) / 128, B * N);
+  if (grid.y > 65535) return MSD_ERR_UNSUPPORTED;
+  if (dtype == MSD_DTYPE_BF16)
+    hipLaunchKernelGGL(rot_block_quant_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, rot_t, (unsigned char*)q,
+                       scale, x_sb, x_sn, x_ss, N, S);
+  else
+    hipLaunchKernelGGL(rot_block_quant_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, rot_t, (unsigned char*)q,
+                       scale, x_sb, x_sn, x_ss, N, S);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 

@@ -32,6 +32,7 @@ SIGNATURES = {
     "mindiesd_mask_to_index": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_int, c_p]),
     "mindiesd_lpt_order": (c_int, [c_p, c_p, c_int, c_int, c_p]),
     "mindiesd_fa_block_quant": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_int, c_p]),
+    "mindiesd_fa_rot_block_quant": (c_int, [c_p, c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_p]),
     "mindiesd_fp8_v_quant_workspace_size": (c_sz, [c_int, c_int]),
     "mindiesd_fp8_v_quant": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_p, c_sz, c_p]),
     "mindiesd_fp8_attention_fwd": (c_int, [c_p] * 7 + [c_int] * 6 + [c_ll] * 3 + [c_f, c_p]),

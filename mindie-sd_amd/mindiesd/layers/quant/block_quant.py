@@ -29,6 +29,29 @@ def _block_quant(x, block_size, layout):
     return q, scale
 
 
+def _rot_block_quant(x, rot, layout):
+    """(x @ rot) rounded to x.dtype, then quantised per (head, 128 tokens) in one pass over x.
+    x 4-D bf16/fp16 GPU tensor in ``layout``, rot [128, 128]; returns (uint8 codes [B,N,S,D], fp32 scale
+    [B,N,ceil(S/128)])."""
+    if x.dtype not in _native.DTYPE_CODE or not x.is_cuda:
+        raise ParametersInvalid(f"fa block quant needs a bf16/fp16 GPU tensor, but got {x.dtype} on {x.device}.")
+    if x.shape[-1] != HEAD_DIM or tuple(rot.shape) != (HEAD_DIM, HEAD_DIM):
+        raise ParametersInvalid(f"rotation + block quant supports head_dim == {HEAD_DIM} and a [{HEAD_DIM}, {HEAD_DIM}] "
+                                f"rotation, but got {x.shape[-1]} and {tuple(rot.shape)}.")
+    ok = x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+    x = x if ok else x.contiguous()
+    rot_t = rot.to(device=x.device, dtype=x.dtype).t().contiguous()
+    b, n, s = (x.shape[0], x.shape[1], x.shape[2]) if layout == "BNSD" else (x.shape[0], x.shape[2], x.shape[1])
+    q = torch.empty((b, n, s, HEAD_DIM), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((b, n, (s + 127) // 128), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _native.lib().mindiesd_fa_rot_block_quant(x.data_ptr(), rot_t.data_ptr(), q.data_ptr(), scale.data_ptr(),
+                                                       _native.DTYPE_CODE[x.dtype], b, n, s, HEAD_DIM,
+                                                       *_strides_bns(x, layout), _native.stream_ptr(x.device))
+    _native.check(rc, "mindiesd_fa_rot_block_quant")
+    return q, scale
+
+
 def fa_block_quant_preprocess(input_tensor, block_size=128, dst_type=torch.float8_e4m3fn, **kwargs):
     """Quantise q, k or v for FP8 attention.  ``layout`` kwarg: 'BNSD' (default) or 'BSND'.
 

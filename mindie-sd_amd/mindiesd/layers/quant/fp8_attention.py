@@ -9,7 +9,7 @@ import torch
 from ... import _native
 from ...utils.exception import ParametersInvalid
 from ..flash_attn.hip_flash_attn import HEAD_DIM, _strides_bns
-from .block_quant import _block_quant
+from .block_quant import _block_quant, _rot_block_quant
 
 
 def quantize_v_per_channel(value, layout="BNSD"):
@@ -49,8 +49,10 @@ def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_d
     return out
 
 
-def fp8_attention_forward(query, key, value, scale=None, layout="BNSD"):
-    """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``."""
+def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None):
+    """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``.
+    ``q_rot`` / ``k_rot`` ([128, 128]): query @ q_rot and key @ k_rot are formed inside the quantisation
+    pass (the rotated tensors are never written)."""
     for name, t in (("query", query), ("key", key), ("value", value)):
         if not isinstance(t, torch.Tensor) or t.dim() != 4:
             raise ParametersInvalid(f"The input {name} must be a 4-D torch.Tensor.")
@@ -64,7 +66,7 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD"):
         raise ParametersInvalid("fp8 attention needs the same batch and head count for query and key/value.")
     if scale is None:
         scale = query.shape[-1] ** -0.5
-    q8, qs = _block_quant(query, 128, layout)
-    k8, ks = _block_quant(key, 128, layout)
+    q8, qs = _block_quant(query, 128, layout) if q_rot is None else _rot_block_quant(query, q_rot, layout)
+    k8, ks = _block_quant(key, 128, layout) if k_rot is None else _rot_block_quant(key, k_rot, layout)
     v8t, vs = quantize_v_per_channel(value, layout)
     return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout)

@@ -32,9 +32,9 @@ class FP8RotateQuantFA(nn.Module):
         layout = kwargs.get("layout", "BNSD")
         if layout not in ("BNSD", "BSND"):
             raise ValueError(f"Unsupported layout: {layout}, expected 'BNSD' or 'BSND'.")
-        query = torch.matmul(query, self.q_rot)
-        key = torch.matmul(key, self.k_rot)
-        return fp8_attention_forward(query, key, value, scale=query.shape[-1] ** -0.5, layout=layout)
+        # the two rotations (torch.matmul in the reference, layer.py:284-285) run inside the quantisation pass
+        return fp8_attention_forward(query, key, value, scale=query.shape[-1] ** -0.5, layout=layout,
+                                     q_rot=self.q_rot, k_rot=self.k_rot)
 
 
 class W8A8MXFP8QuantLinear(nn.Module):

@@ -79,6 +79,14 @@ def dynamic_block_quant(x, row_block=128, col_block=128):
     return torch.from_numpy(codes), torch.from_numpy(scale)
 
 
+def rot_block_quant(x, rot, row_block=128):
+    """FP8RotateQuantFA's first two steps (mindiesd/quantization/layer.py:284-296) on the CPU:
+    ``torch.matmul(x, rot)`` in the 16-bit input type (fp32 accumulation, one rounding), then
+    ``dynamic_block_quant`` over (row_block tokens x all channels)."""
+    y = torch.matmul(x.float(), rot.to(x.dtype).float()).to(x.dtype)
+    return dynamic_block_quant(y, row_block, x.shape[-1])
+
+
 def dequant_block(codes, scale, row_block=128, col_block=128):
     q = torch.from_numpy(e4m3_decode(codes.numpy()))
     s, d = q.shape[-2:]

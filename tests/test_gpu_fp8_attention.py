@@ -90,6 +90,37 @@ def test_fp8_attention_vs_oracle(cuda, layout, s):
     assert err.max() < 0.2 * want.float().abs().max()
 
 
+@pytest.mark.parametrize("layout,dtype", [("BNSD", torch.bfloat16), ("BSND", torch.bfloat16), ("BNSD", torch.float16)])
+def test_rotation_fused_into_block_quant(cuda, layout, dtype):
+    """x @ rot -> 16-bit -> block quantisation in one kernel vs matmul + quantisation on the CPU.  The two
+    sides sum the 128 products of an element in different orders, so a rounded value may now and then land
+    on the neighbouring 16-bit number: scales within one 16-bit ulp, at least 99.5 % of the codes identical,
+    the rest one code step apart."""
+    from mindiesd.layers.quant.block_quant import _rot_block_quant
+    g = torch.Generator().manual_seed(21)
+    rot, _ = torch.linalg.qr(torch.randn(128, 128, generator=g))
+    rot = rot.to(dtype)
+    x = _outlier_inputs((2, 3, 333, 128), seed=22)[0].to(dtype)
+    want_c, want_s = oq.rot_block_quant(x, rot, 128)
+    xin = x if layout == "BNSD" else x.transpose(1, 2).contiguous()
+    codes, scale = _rot_block_quant(xin.to(cuda), rot.to(cuda), layout)
+    codes, scale = codes.cpu(), scale.cpu()
+    assert codes.shape == (2, 3, 333, 128) and scale.shape == (2, 3, 3)
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert torch.allclose(scale, want_s.reshape(2, 3, 3), rtol=2 * ulp, atol=0)
+    same = (codes == want_c)
+    assert same.float().mean() >= 0.995, same.float().mean()
+    diff = (torch.from_numpy(oq.e4m3_decode(codes.numpy())) - torch.from_numpy(oq.e4m3_decode(want_c.numpy()))).abs()
+    step = torch.from_numpy(oq.e4m3_decode(want_c.numpy())).abs().clamp(min=2.0 ** -6) * 2.0 ** -3
+    assert bool((diff <= 1.01 * step).all())
+    # identity rotation: exactly the plain block quantisation
+    from mindiesd.layers.quant.block_quant import _block_quant
+    eye = torch.eye(128, dtype=dtype)
+    c1, s1 = _rot_block_quant(xin.to(cuda), eye.to(cuda), layout)
+    c0, s0 = _block_quant(xin.to(cuda), 128, layout)
+    assert torch.equal(c1, c0) and torch.equal(s1, s0)
+
+
 def test_fp8_rotate_quant_fa_module(cuda):
     """The reference's module shape (mindiesd/quantization/layer.py:274-324): orthogonal rotations
     leave q.k unchanged, so the output must stay close to unquantised attention."""
