@@ -89,6 +89,36 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
                                         float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
                                         const int* order, hipStream_t stream);
 
+/* ---- adaptive block-sparse attention (mask estimate + attention) ------------------------------------------
+ * Block-sparse attention as above (queries and keys of equal length S) with an optional causal mask inside
+ * the selected blocks: key j is visible to query i iff j <= i.  Replaces aclnnAdaBlockSparseAttention behind
+ * torch.ops.mindiesd.ada_block_sparse_attention (csrc/plugin/ada_block_sparse_attention.cpp:27-57); the
+ * int8 sparse_mask is turned into lists with mindiesd_mask_to_index first. */
+int mindiesd_ada_block_sparse_attention_fwd(const void* q, const void* k, const void* v, void* out, int dtype,
+                                            int B, int N, int Nkv, int S, int D,
+                                            long long q_sb, long long q_sn, long long q_ss,
+                                            long long k_sb, long long k_sn, long long k_ss,
+                                            long long v_sb, long long v_sn, long long v_ss,
+                                            long long o_sb, long long o_sn, long long o_ss,
+                                            float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                            int causal, hipStream_t stream);
+
+/* Mask estimate, steps 2 and 3 of aclnnSparseBlockEstimate (csrc/plugin/sparse_block_estimate.cpp:27-85,
+ * csrc/ops/sparse_block_estimate/op_kernel/sparse_block_estimate.h; numpy statement
+ * tests/plugin/test_sparseblockestimate.py:49-145).  Step 1, the strided anti-diagonal score matrix
+ * P'[i][j] = sum_{s<8} q[8i+7-s] . k[8j+s], is a plain [Sr, 8D] x [8D, Sr] GEMM (Sr = ceil(S/8)) that the
+ * caller computes with a GEMM library and passes as pmat [BN][Sr][ldp] (16-bit, ldp % 8 == 0).
+ * mindiesd_sbe_block_scores: scores[bn][I][J] = sum over the 16 x 16 block (I, J) of softmax_j(scale * P'),
+ *   fp32 [BN][NB][NB], NB = ceil(Sr / 16).
+ * mindiesd_sbe_select: per row, key blocks in descending score order (the last block left out) are kept
+ *   until their running sum reaches threshold * total, at most row_sparse * NB of them; the first block is
+ *   kept if keep_sink, the last if keep_recent.  mask int8 [BN][NB][pitch] (pitch >= NB, zero padded; the
+ *   reference uses pitch = NB rounded up to 32), count int32 [BN][NB]. */
+int mindiesd_sbe_block_scores(const void* pmat, float* scores, int dtype, int BN, int Sr, int ldp, float scale,
+                              hipStream_t stream);
+int mindiesd_sbe_select(const float* scores, signed char* mask, int* count, int BN, int NB, int pitch,
+                        float threshold, float row_sparse, int keep_sink, int keep_recent, hipStream_t stream);
+
 /* ---- RainFusion2.0 mask pipeline ---------------------------------------------------------------------
  * Token permutation into 8x8 spatial windows (+ optional block mean pooling) of up to three tensors
  * of one shape; replaces rearrange_with_remaining / avgpool / do_tensor_rearrange_pooling /

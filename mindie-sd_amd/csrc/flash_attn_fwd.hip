@@ -884,6 +884,31 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1>(p, stream);
 }
 
+// Block-sparse attention with an optional causal mask inside the selected blocks (queries and keys of equal
+// length: key j is visible to query i iff j <= i).
+int mindiesd_ada_block_sparse_attention_fwd(const void* q, const void* k, const void* v, void* out, int dtype, int B,
+                                            int N, int Nkv, int S, int D, long long q_sb, long long q_sn,
+                                            long long q_ss, long long k_sb, long long k_sn, long long k_ss,
+                                            long long v_sb, long long v_sn, long long v_ss, long long o_sb,
+                                            long long o_sn, long long o_ss, float scale, const int* blk_idx,
+                                            const int* blk_cnt, int kb_stride, int causal, hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, S, S, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, nullptr, B, N, Nkv, S, S, st, scale);
+  p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride;
+  p.map_mode = g_map_mode;
+  p.QB = (S + 127) / 128;
+  p.causal = causal ? 1 : 0;
+  if (!causal) {
+    if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
+    return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
+  }
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 1>(p, stream);
+}
+
 // Dense attention with the options the plain entry point leaves out: packed variable-length sequences,
 // a causal mask aligned to the bottom-right corner, a boolean attention mask.  Rows whose keys are all
 // masked give zeros.

@@ -1,8 +1,9 @@
 """``torch.ops.mindiesd.*`` operators of the attention path and their keyword wrappers.
 
 Schemas of ``rainfusionattention`` and ``block_sparse_attention`` are the reference's
-(csrc/plugin/register_ops.cpp:41-45, :62-67); the wrappers mirror mindiesd/layers/_custom_ops.py
-(:124-189, :330-390).  ``flash_attention_fwd`` is the dense kernel as an op."""
+(csrc/plugin/register_ops.cpp:41-45, :62-67), likewise ``ada_block_sparse_attention`` and
+``sparse_block_estimate`` (:46-59); the wrappers mirror mindiesd/layers/_custom_ops.py
+(:124-189, :204-305, :330-390).  ``flash_attention_fwd`` is the dense kernel as an op."""
 from typing import List, Optional, Tuple
 
 import torch
@@ -22,6 +23,18 @@ register_ops.define_op(
     "str q_input_layout='BNSD', str kv_input_layout='BNSD', int num_key_value_heads=1, float scale_value=1.0, "
     "int inner_precise=0, int[]? actual_seq_lengths=None, int[]? actual_seq_lengths_kv=None, "
     "int softmax_lse_flag=0) -> (Tensor, Tensor)")
+register_ops.define_op(
+    "ada_block_sparse_attention",
+    "(Tensor query, Tensor key, Tensor value, Tensor sparse_mask, Tensor sparse_count_table, "
+    "str input_layout='BNSD', int sparse_size=128, int num_heads=1, int num_key_value_heads=1, float scale_value=1, "
+    "bool causal=True, int inner_precise=1, int pre_tokens=214748647, int next_tokens=0, "
+    "int[]? actual_seq_lengths=None, int[]? actual_seq_lengths_kv=None) -> Tensor")
+register_ops.define_op(
+    "sparse_block_estimate",
+    "(Tensor query, Tensor key, int[]? actual_seq_lengths=None, int[]? actual_seq_lengths_kv=None, "
+    "str input_layout='BNSD', int stride=8, int sparse_size=128, int num_heads=1, int num_key_value_heads=1, "
+    "float scale_value=1, float threshold=1, bool causal=True, bool keep_sink=True, bool keep_recent=True, "
+    "float row_sparse=1) -> (Tensor, Tensor)")
 register_ops.define_op(
     "flash_attention_fwd",
     "(Tensor query, Tensor key, Tensor value, float scale_value=1.0, str input_layout='BNSD') -> (Tensor, Tensor)")
@@ -197,3 +210,75 @@ def block_sparse_attention(query, key, value, block_sparse_mask: Optional[torch.
     if actual_seq_lengths_kv is not None:
         kwargs["actual_seq_lengths_kv"] = actual_seq_lengths_kv
     return torch.ops.mindiesd.block_sparse_attention(**kwargs)
+
+
+# ---- adaptive block-sparse attention (mindiesd/layers/_custom_ops.py:204-305) -----------------------------------
+@register_ops.register_device_impl("sparse_block_estimate")
+def _sparse_block_estimate_impl(query, key, actual_seq_lengths=None, actual_seq_lengths_kv=None, input_layout="BNSD",
+                                stride=8, sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0,
+                                threshold=1.0, causal=True, keep_sink=True, keep_recent=True, row_sparse=1.0):
+    from .flash_attn.ada_bsa import sparse_block_estimate as run
+    s = query.shape[2] if input_layout == "BNSD" else query.shape[1]
+    _check_lengths(actual_seq_lengths, s, "sparse_block_estimate")
+    _check_lengths(actual_seq_lengths_kv, s, "sparse_block_estimate")
+    return run(query, key, input_layout, stride, sparse_size, scale_value, threshold, causal, keep_sink, keep_recent,
+               row_sparse)
+
+
+@register_ops.register_mindie_fake_op("sparse_block_estimate")
+def sparse_block_estimate_fake(query, key, actual_seq_lengths=None, actual_seq_lengths_kv=None, input_layout="BNSD",
+                               stride=8, sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0,
+                               threshold=1.0, causal=True, keep_sink=True, keep_recent=True, row_sparse=1.0):
+    b, nq, s = (query.shape[0], query.shape[1], query.shape[2]) if input_layout == "BNSD" else \
+        (query.shape[0], query.shape[2], query.shape[1])
+    nb = (s + sparse_size - 1) // sparse_size
+    return (torch.empty((b, nq, nb, (nb + 31) // 32 * 32), device=query.device, dtype=torch.int8),
+            torch.empty((b, nq, nb), device=query.device, dtype=torch.int32))
+
+
+def sparse_block_estimate(query, key, actual_seq_lengths: Optional[List[int]] = None,
+                          actual_seq_lengths_kv: Optional[List[int]] = None, input_layout: str = "BNSD",
+                          stride: int = 8, sparse_size: int = 128, num_heads: int = 1, num_key_value_heads: int = 1,
+                          scale_value: float = 1.0, threshold: float = 1.0, causal: bool = True,
+                          keep_sink: bool = True, keep_recent: bool = True,
+                          row_sparse: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    return torch.ops.mindiesd.sparse_block_estimate(
+        query=query, key=key, actual_seq_lengths=actual_seq_lengths, actual_seq_lengths_kv=actual_seq_lengths_kv,
+        input_layout=input_layout, stride=stride, sparse_size=sparse_size,
+        num_heads=1 if num_heads is None else num_heads,
+        num_key_value_heads=1 if num_key_value_heads is None else num_key_value_heads, scale_value=scale_value,
+        threshold=threshold, causal=causal, keep_sink=keep_sink, keep_recent=keep_recent, row_sparse=row_sparse)
+
+
+@register_ops.register_device_impl("ada_block_sparse_attention")
+def _ada_block_sparse_attention_impl(query, key, value, sparse_mask, sparse_count_table, input_layout="BNSD",
+                                     sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0, causal=True,
+                                     inner_precise=1, pre_tokens=214748647, next_tokens=0, actual_seq_lengths=None,
+                                     actual_seq_lengths_kv=None):
+    from .flash_attn.ada_bsa import ada_block_sparse_attention as run
+    s = query.shape[2] if input_layout == "BNSD" else query.shape[1]
+    _check_lengths(actual_seq_lengths, s, "ada_block_sparse_attention")
+    _check_lengths(actual_seq_lengths_kv, s, "ada_block_sparse_attention")
+    return run(query, key, value, sparse_mask, sparse_count_table, input_layout, sparse_size, scale_value, causal)
+
+
+@register_ops.register_mindie_fake_op("ada_block_sparse_attention")
+def ada_block_sparse_attention_fake(query, key, value, sparse_mask, sparse_count_table, input_layout="BNSD",
+                                    sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0, causal=True,
+                                    inner_precise=1, pre_tokens=214748647, next_tokens=0, actual_seq_lengths=None,
+                                    actual_seq_lengths_kv=None):
+    return torch.empty_like(query)
+
+
+def ada_block_sparse_attention(query, key, value, sparse_mask, sparse_count_table, input_layout: str = "BNSD",
+                               sparse_size: int = 128, num_heads: int = 1, num_key_value_heads: int = 1,
+                               scale_value: float = 1.0, causal: bool = False, inner_precise: int = 1,
+                               pre_tokens: int = 214748647, next_tokens: int = 214748647,
+                               actual_seq_lengths: Optional[List[int]] = None,
+                               actual_seq_lengths_kv: Optional[List[int]] = None) -> torch.Tensor:
+    return torch.ops.mindiesd.ada_block_sparse_attention(
+        query=query, key=key, value=value, sparse_mask=sparse_mask, sparse_count_table=sparse_count_table,
+        input_layout=input_layout, sparse_size=sparse_size, num_heads=1 if num_heads is None else num_heads,
+        num_key_value_heads=1 if num_key_value_heads is None else num_key_value_heads, scale_value=scale_value,
+        causal=causal, inner_precise=inner_precise, pre_tokens=pre_tokens, next_tokens=next_tokens,
+        actual_seq_lengths=actual_seq_lengths, actual_seq_lengths_kv=actual_seq_lengths_kv)

@@ -5,6 +5,7 @@ import torch
 
 from . import rainfusion as rf
 from .hip_flash_attn import flash_attention
+from .sparse_flash_attn_ada_bsa import ada_block_sparse_attention, get_estimate_mask
 from ...utils.exception import ParametersInvalid
 
 
@@ -25,7 +26,9 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_mas
 
     ``sparse_type``: None = dense flash attention; 'rf_v2' / 'rf_v3' = RainFusion2.0 block sparsity
     (index-list and int8-mask variants; both need ``latent_shape_q`` = (t, h, w) with
-    t*h*w + txt_len == S, ``block_size`` 128 and ``sparsity`` in [0, 1)); 'ada_bsa' is not built yet.
+    t*h*w + txt_len == S, ``block_size`` 128 and ``sparsity`` in [0, 1)); 'ada_bsa' = adaptive block
+    sparsity (mask estimated from strided anti-diagonal scores, ``cdf_threshold``, ``sparsity`` as the cap,
+    ``keep_sink`` / ``keep_recent``; non-causal estimation only).
     The output has the layout, dtype and token order of ``q``."""
     check_params(input_layout, sparse_type)
     head_dim = q.shape[-1]
@@ -62,5 +65,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_mas
                                             inner_precise=inner_precise)
         return out
     if sparse_type == "ada_bsa":
-        raise ParametersInvalid("sparse_type 'ada_bsa' is not available in this build.")
+        # sparse_flash_attn.py:151-173 of the reference
+        smask, sct = get_estimate_mask(q, k, v, scale=scale, head_num=head_num, is_causal=is_causal,
+                                       input_layout=input_layout, keep_sink=keep_sink, keep_recent=keep_recent,
+                                       sparsity=sparsity, cdf_threshold=cdf_threshold, sparse_size=block_size)
+        return ada_block_sparse_attention(q, k, v, smask, sct, scale=scale, head_num=head_num, is_causal=is_causal,
+                                          input_layout=input_layout, sparse_size=block_size)
     return flash_attention(q, k, v, scale, input_layout)

@@ -1,0 +1,130 @@
+"""GPU parity of adaptive block-sparse attention vs the CPU oracle.  Mask estimate: the reference's own
+tolerance for its kernel against the numpy statement (tests/plugin/test_sparseblockestimate.py:231-241):
+differing blocks below 2 % of the selected ones, omitted blocks below 1 %.  Attention: the reference's
+kernel rule |err| <= 2^-6 * max(1, |golden|) (tests/plugin/test_adablocksparseattention.py:26-32, :173)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ada_bsa as oab
+from oracle.attention import ref_compare
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(shape, seed, dtype=torch.float16, mul=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * mul).to(dtype)
+
+
+def _structured(shape, seed, dtype):
+    """Scores with structure: a slowly varying component shared by neighbouring tokens plus noise."""
+    b, n, s, d = shape
+    base = _rand((b, n, (s + 63) // 64, d), seed, torch.float32).repeat_interleave(64, dim=2)[:, :, :s]
+    return (base + 0.5 * _rand(shape, seed + 1, torch.float32)).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("s,threshold,row_sparse", [(2048, 0.85, 1.0), (3000, 0.6, 0.5), (1031, 0.9, 1.0)])
+def test_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, dtype):
+    import mindiesd  # noqa: F401
+    q, k = _structured((1, 2, s, 128), 1, dtype), _structured((1, 2, s, 128), 3, dtype)
+    scale = 128 ** -0.5 / 8
+    smask, sct = torch.ops.mindiesd.sparse_block_estimate(
+        q.to(cuda), k.to(cuda), input_layout="BNSD", stride=8, sparse_size=128, num_heads=2, num_key_value_heads=2,
+        scale_value=scale, threshold=threshold, causal=False, keep_sink=True, keep_recent=True, row_sparse=row_sparse)
+    nb = (s + 127) // 128
+    assert smask.shape == (1, 2, nb, (nb + 31) // 32 * 32) and smask.dtype == torch.int8
+    assert sct.shape == (1, 2, nb) and sct.dtype == torch.int32
+    got = smask.cpu().numpy().astype(bool)
+    assert not got[..., nb:].any()
+    assert np.array_equal(sct.cpu().numpy(), got.sum(-1))
+    want = oab.sparse_estimate(q, k, threshold=threshold, force_sparse=row_sparse)
+    got = got[..., :nb]
+    assert got[..., 0].all() and got[..., -1].all()
+    for h in range(2):
+        selected = want[0, h].sum()
+        assert (got[0, h] != want[0, h]).sum() / selected < 0.02
+        assert (got[0, h] < want[0, h]).sum() / selected < 0.01
+
+
+def test_block_scores_and_selection_separately(cuda):
+    from mindiesd.layers.flash_attn.ada_bsa import sparse_block_estimate
+    s = 2500
+    q, k = _structured((1, 1, s, 128), 5, torch.float16), _structured((1, 1, s, 128), 7, torch.float16)
+    mask, cnt, scores = sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=128 ** -0.5 / 8, threshold=0.8,
+                                              row_sparse=0.7, return_scores=True)
+    want = oab.block_scores(q[0, 0].float().numpy(), k[0, 0].float().numpy())
+    got = scores.cpu().numpy()[0, 0]
+    nb = (s + 127) // 128
+    assert got.shape == (nb, nb)
+    # 16-bit products in the logits: block masses agree to a fraction of a percent of a row's mass (16)
+    assert np.abs(got - want).max() < 2e-2 and abs(got.sum() - (s + 7) // 8) < 0.5
+    # the selection kernel on the GPU's own scores reproduces the statement row by row
+    sel = np.stack([oab.select_blocks(got[i], 0.8, 0.7) for i in range(nb)])
+    assert (mask.cpu().numpy()[0, 0, :, :nb].astype(bool) != sel).mean() < 1e-3
+    # switches: without the forced blocks fewer (or equal) blocks are kept
+    m2, c2 = sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=128 ** -0.5 / 8, threshold=0.8, row_sparse=0.7,
+                                   keep_sink=False, keep_recent=False)
+    assert bool((c2 <= cnt).all())
+
+
+@pytest.mark.parametrize("layout", ["BNSD", "BSND"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_ada_block_sparse_attention_vs_oracle(cuda, causal, layout):
+    import mindiesd  # noqa: F401
+    s, nb = 1100, 9
+    q, k, v = _rand((1, 4, s, 128), 9, torch.bfloat16), _rand((1, 2, s, 128), 10, torch.bfloat16), _rand((1, 2, s, 128), 11, torch.bfloat16)
+    g = torch.Generator().manual_seed(12)
+    m = torch.rand(1, 4, nb, nb, generator=g) > 0.5
+    m[:, :, torch.arange(nb), torch.arange(nb)] = True
+    if causal:
+        m &= torch.ones(nb, nb).tril().bool()
+    m[0, 3, 4] = False if not causal else m[0, 3, 4]
+    smask = torch.zeros(1, 4, nb, 32, dtype=torch.int8)
+    smask[..., :nb] = m.to(torch.int8)
+    sct = m.sum(-1).to(torch.int32)
+    want = oab.ada_block_sparse_attention(q, k, v, m.numpy(), causal=causal)
+    args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = torch.ops.mindiesd.ada_block_sparse_attention(
+        *(t.to(cuda) for t in args), smask.to(cuda), sct.to(cuda), input_layout=layout, sparse_size=128, num_heads=4,
+        num_key_value_heads=2, scale_value=128 ** -0.5, causal=causal).cpu()
+    out = out if layout == "BNSD" else out.transpose(1, 2)
+    eb, ok, mx = ref_compare(want, out, 2.0 ** -6)
+    assert ok, (eb, mx)
+    if not causal:
+        assert not out[0, 3, 512:640].any()
+
+
+def test_sparse_attention_front_door_ada_bsa(cuda):
+    from mindiesd import sparse_attention
+    from mindiesd.layers.flash_attn.sparse_flash_attn_ada_bsa import get_estimate_mask
+    s = 2100
+    q, k = _structured((1, 2, s, 128), 13, torch.bfloat16), _structured((1, 2, s, 128), 15, torch.bfloat16)
+    v = _rand((1, 2, s, 128), 17, torch.bfloat16)
+    out = sparse_attention(q.to(cuda), k.to(cuda), v.to(cuda), head_num=2, input_layout="BNSD", sparse_type="ada_bsa",
+                           cdf_threshold=0.8, sparsity=0.3).cpu()
+    smask, _ = get_estimate_mask(q.to(cuda), k.to(cuda), v.to(cuda), scale=128 ** -0.5, head_num=2, cdf_threshold=0.8,
+                                 sparsity=0.3)
+    nb = (s + 127) // 128
+    want = oab.ada_block_sparse_attention(q, k, v, smask.cpu().numpy()[..., :nb].astype(bool))
+    assert ref_compare(want, out, 2.0 ** -6)[1]
+    density = smask.float().sum() / (2 * nb * nb)
+    assert 0.05 < density <= 0.75
+
+
+def test_ada_bsa_errors(cuda):
+    import mindiesd  # noqa: F401
+    q = torch.randn(1, 1, 256, 128, dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.sparse_block_estimate(q, q, input_layout="TND", causal=False)
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.sparse_block_estimate(q, q, stride=4, causal=False)
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.sparse_block_estimate(q, q, causal=True)
+    m = torch.ones(1, 1, 2, 32, dtype=torch.int8, device=cuda)
+    c = torch.full((1, 1, 2), 2, dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.ada_block_sparse_attention(q, q, q, m[:, :, :1], c, causal=False)
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.ada_block_sparse_attention(q, q, q, m, c, sparse_size=64, causal=False)

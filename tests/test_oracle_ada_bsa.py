@@ -1,0 +1,88 @@
+"""Pins of the adaptive block-sparse oracle (oracle/ada_bsa.py): the chunked running-softmax statement of
+the block scores against a direct global softmax, the selection rule on hand-worked rows, and the sparse
+attention against dense / causal attention in the cases where they coincide."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ada_bsa as oab
+from oracle.attention import attention_math
+
+
+def _global_block_scores(q, k, stride=8, reduce=16):
+    d = q.shape[1]
+    sq = -(-q.shape[0] // stride) * stride
+    qp = np.zeros((sq, d), np.float64)
+    qp[:q.shape[0]] = q
+    kp = np.zeros((sq, d), np.float64)
+    kp[:k.shape[0]] = k
+    sr = sq // stride
+    p = np.zeros((sr, sr))
+    for i in range(sr):
+        for s in range(stride):
+            p[i] += qp[stride * i + stride - 1 - s] @ kp[s::stride].T
+    p /= np.sqrt(d) * stride
+    prob = np.exp(p - p.max(-1, keepdims=True))
+    prob /= prob.sum(-1, keepdims=True)
+    nb = -(-sr // reduce)
+    pad = np.zeros((nb * reduce, nb * reduce))
+    pad[:sr, :sr] = prob
+    return pad.reshape(nb, reduce, nb, reduce).sum((1, 3))
+
+
+@pytest.mark.parametrize("s", [128, 1000, 1027, 9000])
+def test_block_scores_equal_global_softmax(s):
+    rng = np.random.RandomState(s)
+    q = rng.standard_normal((s, 8)).astype(np.float32) * 2
+    k = rng.standard_normal((s, 8)).astype(np.float32) * 2
+    got = oab.block_scores(q, k)
+    want = _global_block_scores(q, k)
+    assert got.shape == want.shape == (-(-s // 128), -(-s // 128))
+    assert np.abs(got - want).max() < 2e-5
+    # every strided row carries probability mass 1
+    assert abs(got.sum() - (-(-s // 8))) < 1e-2
+
+
+def test_select_blocks_hand_worked_rows():
+    row = [0.5, 0.2, 0.1, 0.15, 0.05]
+    # ranking without the last block: 0.5 0.2 0.15 0.1 0; total 0.95; 0.6 * 0.95 = 0.57 is passed by the second
+    assert oab.select_blocks(row, 0.6, 1.0).tolist() == [True, True, False, False, True]
+    # without the forced blocks the guard alone decides (0.2): the sink passes it anyway, the last block does not
+    assert oab.select_blocks(row, 0.6, 1.0, keep_sink=False, keep_recent=False).tolist() == [True, True, False, False, False]
+    # threshold 1: everything that carries mass (and, through the zeroed last entry, the rest)
+    assert oab.select_blocks(row, 1.0, 1.0).all()
+    # cap: at most int(0.4 * 5) = 2 ranked blocks although 0.99 asks for 4
+    assert oab.select_blocks(row, 0.99, 0.4).tolist() == [True, True, False, False, True]
+    # a sink that would not make it on its own is forced
+    assert oab.select_blocks([0.01, 0.6, 0.3, 0.09], 0.5, 1.0).tolist() == [True, True, False, True]
+    # ties: stable order, both tied blocks pass the guard
+    assert oab.select_blocks([0.3, 0.3, 0.3, 0.1], 0.4, 1.0).tolist() == [True, True, True, True]
+
+
+def test_sparse_estimate_invariants():
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, 2, 1100, 32, generator=g)
+    k = torch.randn(1, 1, 1100, 32, generator=g)
+    m = oab.sparse_estimate(q, k, threshold=0.7, force_sparse=0.5)
+    assert m.shape == (1, 2, 9, 9) and m[..., 0].all() and m[..., -1].all()
+    assert (m.sum(-1) <= int(0.5 * 9) + 2).all()
+    assert oab.sparse_estimate(q, k, threshold=1.0, force_sparse=1.0).all()
+    # monotone in the threshold
+    lo, hi = oab.sparse_estimate(q, k, threshold=0.3), oab.sparse_estimate(q, k, threshold=0.9)
+    assert (hi | ~lo).all()
+
+
+def test_ada_attention_reduces_to_dense_and_causal():
+    g = torch.Generator().manual_seed(1)
+    q, k, v = (torch.randn(1, 2, 300, 16, generator=g) for _ in range(3))
+    full = np.ones((1, 2, 3, 3), dtype=bool)
+    dense = attention_math(q, k, v, None, 16 ** -0.5, head_first=True)
+    assert torch.allclose(oab.ada_block_sparse_attention(q, k, v, full, blocksize=128), dense, atol=1e-5)
+    tril = np.tril(np.ones((3, 3), dtype=bool))[None, None].repeat(2, axis=1)
+    causal = attention_math(q, k, v, torch.ones(300, 300).tril().bool(), 16 ** -0.5, head_first=True)
+    assert torch.allclose(oab.ada_block_sparse_attention(q, k, v, tril, causal=True, blocksize=128), causal, atol=1e-5)
+    # an empty row gives zeros; grouped-query heads share keys
+    m = full.copy()
+    m[0, 1, 2] = False
+    out = oab.ada_block_sparse_attention(q, k[:, :1], v[:, :1], m, blocksize=128)
+    assert not out[0, 1, 256:].any() and out[0, 0].abs().sum() > 0
