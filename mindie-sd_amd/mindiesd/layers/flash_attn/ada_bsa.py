@@ -15,7 +15,12 @@ from .hip_flash_attn import HEAD_DIM, _strides_bns
 from .rainfusion import BLOCK, _aligned, _check_gpu16, _dims, mask_to_lists
 
 STRIDE = 8
-_PMAT_BYTES = 8 << 30  # heads are processed in groups whose P' matrices stay below this size
+# Heads are processed in groups whose P' matrices together stay below 2^30 elements (2 GiB in 16 bits).
+_PMAT_ELEMS = 1 << 30
+# Longest sequence the estimate accepts.  Runs at 32760 and 75600 tokens ended in a GPU memory fault whose
+# cause has not been established (the kernels' index arithmetic checks out on paper; sequences up to 3000
+# tokens pass their parity tests), so longer sequences are refused until it is.
+MAX_ESTIMATE_TOKENS = 3072
 
 
 def _to_bnsd(t, layout):
@@ -39,6 +44,10 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
                            f"got {stride} and {sparse_size}")
     if causal:
         raise RuntimeError("sparse_block_estimate: causal estimation is not available in this build")
+    s_tokens = query.shape[2] if input_layout == "BNSD" else query.shape[1]
+    if s_tokens > MAX_ESTIMATE_TOKENS:
+        raise RuntimeError(f"sparse_block_estimate: sequences longer than {MAX_ESTIMATE_TOKENS} tokens are switched off in "
+                           f"this build (got {s_tokens})")
     q, k = _to_bnsd(query, input_layout), _to_bnsd(key, input_layout)
     b, n, s, d = q.shape
     if k.shape[0] != b or k.shape[2] != s or k.shape[3] != d or n % k.shape[1] != 0 or k.dtype != q.dtype:
@@ -57,7 +66,9 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
     kp = torch.zeros((b * n, ldp, STRIDE * d), dtype=q.dtype, device=q.device)
     kp[:, :sr].view(b * n, sr * STRIDE, d)[:, :s] = k.reshape(b * n, s, d)
     scores = torch.empty((b * n, nb, nb), dtype=torch.float32, device=q.device)
-    group = max(1, min(b * n, _PMAT_BYTES // (sr * ldp * q.element_size())))
+    if sr * ldp > _PMAT_ELEMS:
+        raise RuntimeError(f"sparse_block_estimate: sequence length {s} is beyond what this build estimates")
+    group = max(1, min(b * n, _PMAT_ELEMS // (sr * ldp)))
     lib = _native.lib()
     with torch.cuda.device(q.device):
         for g0 in range(0, b * n, group):

@@ -113,6 +113,16 @@ def test_sparse_attention_front_door_ada_bsa(cuda):
     assert 0.05 < density <= 0.75
 
 
+@pytest.mark.skip(reason="the estimate at 32760 tokens (B1 N12) and 75600 tokens (B1 N40) ended in a GPU memory fault "
+                         "whose cause is not established; sequences beyond 3072 tokens are refused by the host code")
+def test_sparse_block_estimate_long_sequences(cuda):
+    from mindiesd.layers.flash_attn import ada_bsa
+    q = _structured((1, 12, 32760, 128), 21, torch.bfloat16).to(cuda)
+    k = _structured((1, 12, 32760, 128), 23, torch.bfloat16).to(cuda)
+    mask, cnt = ada_bsa.sparse_block_estimate(q, k, scale_value=128 ** -0.5 / 8, threshold=0.9, row_sparse=0.25)
+    assert mask.shape == (1, 12, 256, 256) and int(cnt.min()) >= 2
+
+
 def test_ada_bsa_errors(cuda):
     import mindiesd  # noqa: F401
     q = torch.randn(1, 1, 256, 128, dtype=torch.float16, device=cuda)
@@ -122,6 +132,9 @@ def test_ada_bsa_errors(cuda):
         torch.ops.mindiesd.sparse_block_estimate(q, q, stride=4, causal=False)
     with pytest.raises(RuntimeError):
         torch.ops.mindiesd.sparse_block_estimate(q, q, causal=True)
+    big = torch.zeros(1, 1, 3073, 128, dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="switched off"):
+        torch.ops.mindiesd.sparse_block_estimate(big, big, causal=False)
     m = torch.ones(1, 1, 2, 32, dtype=torch.int8, device=cuda)
     c = torch.full((1, 1, 2), 2, dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError):
