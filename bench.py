@@ -30,9 +30,9 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes of one dense 14B-720p launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by a 1 GiB copy kernel (summary and commands: profiles/fa_fwd_dense_bf16_wan14b_720p.md)
-DENSE_TRAFFIC_BYTES = 2.11e10
+DENSE_TRAFFIC_BYTES = 7.10e10
 
-# workloads (BASELINE.json configs)
+# workloads
 CFG_14B_720P = dict(B=1, N=40, S=75600, D=128, grid=(21, 45, 80))
 CFG_1P3B = dict(B=1, N=12, S=32760, D=128, grid=(21, 30, 52))
 CFG_14B_480P = dict(B=1, N=40, S=32760, D=128, grid=(21, 30, 52))
@@ -199,6 +199,15 @@ def extra_sparse(device, steps, warmup, dense_ms):
                                                           keep_diagonal=True), steps, warmup)
     perm_ms, _ = time_steps(lambda: rf.do_tensor_rearrange_pooling(q, k, v, 0, 128, cfg["grid"], cfg["grid"], "BNSD"),
                             steps, warmup)
+    # the same pipeline with the top 25 % of the key blocks alone (no forced first-frame / diagonal blocks)
+    args25 = dict(latent_shape_q=cfg["grid"], sparsity=0.75, input_layout="BNSD", keep_diagonal=False,
+                  protect_first_frame=False)
+    out, mask25 = rf.bsa_sparse_attention_v3(q, k, v, **args25)
+    density25 = float(mask25.float().mean())
+    full25_ms, _ = time_steps(lambda: rf.bsa_sparse_attention_v3(q, k, v, **args25), steps, warmup)
+    idx25, cnt25 = rf.mask_to_lists(mask25)
+    kern25_ms, _ = time_steps(lambda: rf.block_sparse_attention_lists(q_, k_, v_, idx25, cnt25, cfg["D"] ** -0.5,
+                                                                      "BNSD"), steps, warmup)
     del out
     torch.cuda.empty_cache()
     f = attn_flops(cfg)
@@ -212,6 +221,10 @@ def extra_sparse(device, steps, warmup, dense_ms):
         "attention_kernel_speedup_vs_dense": dense_ms / km,
         "permute_pool_ms": median(perm_ms), "permute_pool_gbs": 6 * 774.144e6 / median(perm_ms) / 1e6,
         "mask_ms": median(mask_ms),
+        "topk_only_mask_density": density25,
+        "topk_only_pipeline_ms": median(full25_ms), "topk_only_speedup_vs_dense": dense_ms / median(full25_ms),
+        "topk_only_attention_kernel_ms": median(kern25_ms),
+        "topk_only_attention_kernel_speedup_vs_dense": dense_ms / median(kern25_ms),
     }
 
 

@@ -83,6 +83,27 @@ __device__ __forceinline__ s16x4_t lds_read_tr16(const void* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)(uintptr_t)(p));
 }
 
+// The same read written as inline asm, for loops that keep LDS-DMA requests in flight: the compiler orders
+// the builtin after every LDS-DMA still outstanding (it waits for vmcnt(0)), which would make each tile wait
+// for the whole next tile before its first V read.  The asm form carries no such dependence; in exchange the
+// compiler does not know that the result arrives later, so the caller must pass the registers through
+// lds_wait_tr<N>() (s_waitcnt lgkmcnt(N), N = number of LDS reads issued after them that may stay in
+// flight) before using them.
+template <int OFFSET>
+__device__ __forceinline__ s16x4_t lds_read_tr16_async(unsigned lds_addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "ds offset field is 16 bits");
+  s16x4_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_addr), "n"(OFFSET));
+  return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_tr(s16x4_t (&r)[8]) {
+  static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit counter");
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
+               : "n"(N));
+}
+
 // Combine a value with the one held by the lane 32 positions away (the other half of the
 // wavefront) using v_permlane32_swap: after the swap one result register holds lanes 0..31 of
 // the input in both halves and the other holds lanes 32..63 in both halves.

@@ -21,6 +21,7 @@
 //     K tile [key][128]: 16-byte chunk c of row key is stored at chunk c ^ (key & 15)
 //     V tile [key][128]: 64-byte chunk c of row key is stored at chunk c ^ (key & 3)
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 
@@ -75,6 +76,16 @@ struct FaCfg {
 };
 
 #if defined(__HIP_DEVICE_COMPILE__)
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
 // LDS-DMA of one K tile and one V tile: every wave issues G pairs of 1 KiB transfers.
 template <int G, int NWAVES>
 __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu_buffer_rsrc_t v_rsrc,
@@ -222,6 +233,11 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int v_key = 4 * h + ((lane & 15) >> 2);  // key & 3 == ((lane&15)>>2) for every base key (multiples of 4)
   const int v_row_off = v_key * C::kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
   const int v_swz = (lane & 15) >> 2;
+  // LDS byte address of this lane's V^T read for head_dim block db of the tile in stage 0, key step 0
+  unsigned v_lds[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+    v_lds[db] = (unsigned)(uintptr_t)smem + C::kTileBytes + v_row_off + ((db ^ v_swz) << 6);
 
   // ---- stream state (all wave-uniform) -----------------------------------------------------------
   // Block lists live in registers, 64 ids per batch (one per lane); the next batch is requested when
@@ -432,6 +448,43 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------------------
+    // 128-key tiles: V^T fragments are read one 16-key step ahead of the matrix instructions that use them
+    // with asm reads and explicit waits (see lds_read_tr16_async), so that the next tile's LDS-DMA stays in
+    // flight until the end of the tile.  With 64-key tiles (two workgroups per CU cover each other's stalls)
+    // the builtin and the compiler's own schedule measured faster.
+    if constexpr (BN == 128) {
+      constexpr int kSteps = C::kNKB * 2;
+      s16x4_t vf[2][8];
+      auto issue = [&](auto step_c, s16x4_t(&dst)[8]) __attribute__((always_inline)) {
+        constexpr int s = decltype(step_c)::value;
+        constexpr int off = ((s >> 1) * 32 + (s & 1) * 16) * C::kRowBytes;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const unsigned a = v_lds[db] + stage * C::kStageBytes;
+          dst[2 * db] = lds_read_tr16_async<off>(a);
+          dst[2 * db + 1] = lds_read_tr16_async<off + 8 * C::kRowBytes>(a);
+        }
+      };
+      issue(std::integral_constant<int, 0>{}, vf[0]);
+      static_for<kSteps>([&](auto step_c) __attribute__((always_inline)) {
+        constexpr int s = decltype(step_c)::value;
+        if constexpr (s + 1 < kSteps) {
+          issue(std::integral_constant<int, s + 1>{}, vf[(s + 1) & 1]);
+          lds_wait_tr<8>(vf[s & 1]);
+        } else {
+          lds_wait_tr<0>(vf[s & 1]);
+        }
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          union { s16x4_t s2[2]; X8 x; } u;
+          u.s2[0] = vf[s & 1][2 * db];
+          u.s2[1] = vf[s & 1][2 * db + 1];
+#pragma unroll
+          for (int qb = 0; qb < C::kNQB; ++qb)
+            oacc[db][qb] = E::mfma32(u.x, pf[qb][s >> 1][s & 1], oacc[db][qb]);
+        }
+      });
+    } else {
 #pragma unroll
     for (int kb = 0; kb < C::kNKB; ++kb) {
 #pragma unroll
@@ -450,6 +503,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
           for (int qb = 0; qb < C::kNQB; ++qb) oacc[db][qb] = E::mfma32(u.x, pf[qb][kb][t2], oacc[db][qb]);
         }
       }
+    }
     }
 
       first = false;

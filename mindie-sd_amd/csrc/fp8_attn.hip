@@ -383,9 +383,16 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   __builtin_amdgcn_s_waitcnt(0x0f70);
   __syncthreads();
 
+  // The K scale of a tile is fetched one tile ahead and BEFORE that step's LDS-DMA requests: memory
+  // operations complete in order, so a scale requested after them could only be used once the whole next
+  // tile has landed, which would put that wait into the middle of every tile.
+  float k_sc_cur = n_tiles > 0 ? k_sc[0] : 0.f;
   auto tile_step = [&](const int t, auto stage_c) {
     constexpr int stage = decltype(stage_c)::value;
-    if (t + 1 < n_tiles) load_tile(t + 1, stage ^ 1);
+    const float k_sc_next = k_sc[t + 1 < n_tiles ? t + 1 : t];
+    // issued after the last tile as well (past the end of the buffers: reads as zeros, nobody uses it), so that
+    // the number of requests in flight behind the scale is the same on every path
+    load_tile(t + 1, stage ^ 1);
     MSD_LDS const char* kb_base = smem + stage * kStage;
     MSD_LDS const char* vb_base = kb_base + kTile;
 
@@ -417,7 +424,8 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     }
 
     // ---- online softmax (exp2 domain, lazily moved reference maximum), P -> E4M3 -------------------------------
-    const float c = q_sc * k_sc[t];  // dequantisation scales of this tile folded into the softmax scale
+    const float c = q_sc * k_sc_cur;  // dequantisation scales of this tile folded into the softmax scale
+    k_sc_cur = k_sc_next;
     float mx = sacc[0][0];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
