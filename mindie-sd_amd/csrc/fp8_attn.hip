@@ -96,6 +96,48 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsign
 #endif
 }
 
+// The same for 128-token blocks with the block held in registers: a thread requests its 8 rows x 8 channels
+// at once (more requests in flight than the row loop above) and quantises them without a second read.
+template <int DT>
+__global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, unsigned char* q, float* scale,
+                                                             long long sb, long long sn, long long ss, int N, int S) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using T = typename Elem<DT>::type;
+  __shared__ float red[4];
+  const int blk = blockIdx.x, bn = blockIdx.y;
+  const int b = bn / N, n = bn - b * N;
+  const int nblk = gridDim.x;
+  const T* x = (const T*)x_ + b * sb + n * sn;
+  const int row0 = blk * 128, rows = min(128, S - row0);
+  const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
+  union { i32x4_t v; T e[8]; } u[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = rgrp + 16 * i;
+    u[i].v = i32x4_t{0, 0, 0, 0};
+    if (r < rows) u[i].v = *(const i32x4_t*)(x + (long long)(row0 + r) * ss + c16 * 8);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf((float)u[i].e[j]));
+  amax = block_max_256(amax, red);
+  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  if (threadIdx.x == 0) scale[(long long)bn * nblk + blk] = sc;
+  unsigned char* qo = q + ((long long)bn * S + row0) * 128 + c16 * 8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = rgrp + 16 * i;
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn((float)u[i].e[j], sc);
+    const i32x2_t w = {pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
+    if (r < rows) *(i32x2_t*)(qo + (long long)r * 128) = w;
+  }
+#endif
+}
+
 // ---- rotation + block quantisation in one pass ------------------------------------------------------------------
 // y = x @ R (R a fixed [128][128] matrix, e.g. a Hadamard rotation that spreads outliers over the channels),
 // y rounded to the 16-bit input type as a separate matmul would leave it, then quantised like
@@ -223,14 +265,14 @@ __host__ __device__ __forceinline__ int v8t_pos(int kk) {
 }
 
 // V [B][N][S][128] -> V8T [B][N][128][S128] bytes + per-channel scale [B][N][128] = amax/448.
-// One workgroup = 64 keys of one (batch, head).
+// One workgroup = 128 keys of one (batch, head): every channel row it writes is one full 128-byte line.
 template <int DT>
 __global__ __launch_bounds__(256) void v_quant_transpose_kernel(const void* v_, const unsigned* amax_bits,
                                                                 unsigned char* v8t, float* vscale, long long sb,
                                                                 long long sn, long long ss, int N, int S, int S128) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using T = typename Elem<DT>::type;
-  __shared__ unsigned char tile[128][64 + 16];  // [channel][position], padded rows
+  __shared__ __attribute__((aligned(16))) unsigned char tile[128][128 + 16];  // [channel][position], padded rows
   const int grp = blockIdx.x, bn = blockIdx.y, b = bn / N, n = bn - b * N;
   const T* v = (const T*)v_ + b * sb + n * sn;
   const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
@@ -244,30 +286,32 @@ __global__ __launch_bounds__(256) void v_quant_transpose_kernel(const void* v_, 
 #pragma unroll
     for (int j = 0; j < 8; ++j) vscale[(long long)bn * 128 + c16 * 8 + j] = sc[j];
   }
-  for (int kk = rgrp; kk < 64; kk += 16) {
-    const int key = grp * 64 + kk;
-    float f[8];
-    if (key < S) {
-      load8<DT>(v + (long long)key * ss + c16 * 8, f);
-    } else {
+  // all 8 rows of this thread are requested before the first one is used
+  union { i32x4_t v; T e[8]; } u[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) f[j] = 0.f;
-    }
-    const int pos = v8t_pos(kk);
+  for (int i = 0; i < 8; ++i) {
+    const int key = grp * 128 + rgrp + 16 * i;
+    u[i].v = i32x4_t{0, 0, 0, 0};
+    if (key < S) u[i].v = *(const i32x4_t*)(v + (long long)key * ss + c16 * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int kk = rgrp + 16 * i;
+    const int pos = (kk & 64) + v8t_pos(kk & 63);
 #pragma unroll
     for (int j = 0; j < 8; j += 4) {
-      const int w = pack4_e4m3(__fdiv_rn(f[j], sc[j]), __fdiv_rn(f[j + 1], sc[j + 1]), __fdiv_rn(f[j + 2], sc[j + 2]),
-                               __fdiv_rn(f[j + 3], sc[j + 3]));
+      const int w = pack4_e4m3(__fdiv_rn((float)u[i].e[j], sc[j]), __fdiv_rn((float)u[i].e[j + 1], sc[j + 1]),
+                               __fdiv_rn((float)u[i].e[j + 2], sc[j + 2]), __fdiv_rn((float)u[i].e[j + 3], sc[j + 3]));
 #pragma unroll
       for (int e = 0; e < 4; ++e) tile[c16 * 8 + j + e][pos] = (unsigned char)((unsigned)w >> (8 * e));
     }
   }
   __syncthreads();
-  // 128 channel rows x 64 bytes: 4 lanes write one row
-  for (int i = threadIdx.x; i < 128 * 4; i += 256) {
-    const int ch = i >> 2, part = i & 3;
+  // 128 channel rows x 128 bytes: 8 lanes write one row
+  for (int i = threadIdx.x; i < 128 * 8; i += 256) {
+    const int ch = i >> 3, part = i & 7;
     const i32x4_t w = *(const i32x4_t*)&tile[ch][part * 16];
-    *(i32x4_t*)(v8t + ((long long)bn * 128 + ch) * S128 + grp * 64 + part * 16) = w;
+    *(i32x4_t*)(v8t + ((long long)bn * 128 + ch) * S128 + grp * 128 + part * 16) = w;
   }
 #endif
 }
@@ -522,6 +566,15 @@ int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
   if (((uintptr_t)x & 15) || ((uintptr_t)q & 7) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
   dim3 grid((S + block_size - 1) / block_size, B * N);
+  if (block_size == 128) {
+    if (dtype == MSD_DTYPE_BF16)
+      hipLaunchKernelGGL(block_quant128_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale,
+                         x_sb, x_sn, x_ss, N, S);
+    else
+      hipLaunchKernelGGL(block_quant128_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale,
+                         x_sb, x_sn, x_ss, N, S);
+    return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+  }
   if (dtype == MSD_DTYPE_BF16)
     hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
                        x_sn, x_ss, N, S, block_size);
@@ -565,7 +618,7 @@ int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, in
   const int S128 = (S + 127) / 128 * 128;
   hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nbits + 255) / 256)), dim3(256), 0, stream, (unsigned*)workspace,
                      0u, nbits);
-  dim3 g1((S + 1023) / 1024, B * N), g2(S128 / 64, B * N);
+  dim3 g1((S + 1023) / 1024, B * N), g2(S128 / 128, B * N);
   if (dtype == MSD_DTYPE_BF16) {
     hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_BF16>, g1, dim3(256), 0, stream, v, (unsigned*)workspace, v_sb, v_sn,
                        v_ss, N, S);
