@@ -165,21 +165,31 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   __syncthreads();
 
   // ---- scores: exact dot -> fp32 -> 16 bit; * scale (fp32) -> 16 bit -----------------------------
+  // 16 lanes share one key block: each reads 16 bytes of its pooled row (one coalesced 256-byte row per group)
+  // and the 16 partial sums are added with lane exchanges.  Every product and sum is exact in fp64, so the order
+  // of summation does not matter.
   float lmax = -INFINITY;
-  for (int c = tid; c < NB; c += 256) {
-    const T* kr = kp + (long long)c * p.p_sblk;
-    double acc = 0.0;
-#pragma unroll 4
-    for (int d0 = 0; d0 < 128; d0 += 8) {
-      union { i32x4_t v; T e[8]; } u;
-      u.v = *(const i32x4_t*)(kr + d0);
+  const int sub = tid & 15, grp16 = tid >> 4;
+  double qd[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc = fma((double)qrow[d0 + j], (double)(float)u.e[j], acc);
+  for (int j = 0; j < 8; ++j) qd[j] = (double)qrow[sub * 8 + j];
+  for (int c0 = 0; c0 < NB; c0 += 16) {
+    const int c = c0 + grp16;
+    double acc = 0.0;
+    if (c < NB) {
+      union { i32x4_t v; T e[8]; } u;
+      u.v = *(const i32x4_t*)(kp + (long long)c * p.p_sblk + sub * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc = fma(qd[j], (double)(float)u.e[j], acc);
     }
-    const float s16 = round16<DT>((float)acc);
-    const float x = round16<DT>(__fmul_rn(s16, p.scale));
-    xs[c] = x;
-    lmax = fmaxf(lmax, x);
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (c < NB) {
+      const float s16 = round16<DT>((float)acc);
+      const float x = round16<DT>(__fmul_rn(s16, p.scale));
+      if (sub == 0) xs[c] = x;
+      lmax = fmaxf(lmax, x);
+    }
   }
   red[tid] = (double)lmax;
   __syncthreads();
