@@ -574,261 +574,6 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-// ---- ping-pong variant (dense) ---------------------------------------------------------------------------
-// Same tiling as fa_fwd_kernel<8 waves x 32 rows, 128-key tiles>, but the two waves that share a SIMD
-// run half an interval apart: between two workgroup barriers, waves 0-3 issue their matrix work
-// (O += P(t) V(t), then S(t+1) = K(t+1) Q^T) and afterwards the softmax of tile t+1, while waves 4-7
-// first run the softmax of tile t and then the same matrix work.  While one wave of a SIMD feeds the
-// matrix pipe the other one keeps the vector ALU busy, instead of both waiting for each other as
-// they do when every wave walks QK^T -> softmax -> PV in lockstep.
-// LDS holds V(t) and K(t+1) for the current interval and receives V(t+1), K(t+2) by LDS-DMA.
-template <int DT>
-__global__ __launch_bounds__(512, 2) void fa_fwd_pp_kernel(const FaParams p) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  using E = Elem<DT>;
-  using T = typename E::type;
-  using X8 = typename E::x8;
-  constexpr int NWAVES = 8, BM = 256, BN = 128, kRowBytes = 256;
-  constexpr int kTileBytes = BN * kRowBytes;  // 32 KiB
-  constexpr int kORowBytes = kRowBytes + 8;
-  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  MSD_LDS char* smem = (MSD_LDS char*)smem_raw;  // [K0 | K1 | V0 | V1]
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l32 = lane & 31;
-  const int h = lane >> 5;
-  const bool late = wave >= 4;  // waves 4-7: softmax first, then matrix work
-
-  const int q_tiles = (p.Sq + BM - 1) / BM;
-  const int total = p.B * p.N * q_tiles;
-  const int per_xcd = (total + 7) / 8;
-  const int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
-  if (work >= total) return;
-  const int bn = work / q_tiles;
-  const int qt = work - bn * q_tiles;
-  const int b = bn / p.N;
-  const int n = bn - b * p.N;
-  const int nkv = n / (p.N / p.Nkv);
-  const int q0 = qt * BM;
-  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
-  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
-  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
-  const int n_tiles = (p.Skv + BN - 1) / BN;
-
-  X8 qf[8];
-  {
-    const int qrow = q0 + wave * 32 + l32;
-    const bool ok = qrow < p.Sq;
-    const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * h;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      X8 v = *(const X8*)(src + 16 * ks);
-      if (!ok) v = X8{0};
-      qf[ks] = v;
-    }
-  }
-  f32x16_t oacc[4];
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-
-  // ---- LDS-DMA: 4 groups of 4 rows per wave and tile --------------------------------------------------
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kg, 0, (int)(((long long)(p.Skv - 1) * p.k_ss + 128) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vg, 0, (int)(((long long)(p.Skv - 1) * p.v_ss + 128) * 2), 0x00020000);
-  const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
-  int k_voff[4], v_voff[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 4 * (i * NWAVES + wave) + (lane >> 4);
-    const int pc = lane & 15;
-    k_voff[i] = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
-    v_voff[i] = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
-  }
-  auto load_k = [&](int t) {
-    MSD_LDS char* dst = smem + (t & 1) * kTileBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(dst + (i * NWAVES + wave) * 1024), 16, k_voff[i],
-                                               t * BN * k_row_bytes, 0, 0);
-  };
-  auto load_v = [&](int t) {
-    MSD_LDS char* dst = smem + (2 + (t & 1)) * kTileBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(dst + (i * NWAVES + wave) * 1024), 16, v_voff[i],
-                                               t * BN * v_row_bytes, 0, 0);
-  };
-
-  const int k_row_off = l32 * kRowBytes;
-  const int k_swz = l32 & 15;
-  const int v_key = 4 * h + ((lane & 15) >> 2);
-  const int v_row_off = v_key * kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
-  const int v_swz = (lane & 15) >> 2;
-
-  f32x16_t sacc[4];
-  X8 pf[4][2];
-
-  // S^T(t) = K(t) Q^T
-  auto qk = [&](int t) {
-    MSD_LDS const char* kb_base = smem + (t & 1) * kTileBytes;
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-    X8 afrag[2][4];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-      afrag[0][kb] = *(MSD_LDS const X8*)(kb_base + kb * 32 * kRowBytes + k_row_off + ((h ^ k_swz) << 4));
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      if (ks + 1 < 8) {
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-          afrag[(ks + 1) & 1][kb] =
-              *(MSD_LDS const X8*)(kb_base + kb * 32 * kRowBytes + k_row_off + (((2 * (ks + 1) + h) ^ k_swz) << 4));
-      }
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb) sacc[kb] = E::mfma32(afrag[ks & 1][kb], qf[ks], sacc[kb]);
-    }
-    const int key0 = t * BN;
-    if (key0 + BN > p.Skv) {
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (key0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3) >= p.Skv) sacc[kb][r] = -INFINITY;
-    }
-  };
-  // P^T(t) from S^T(t): online softmax in the exp2 domain with a lazily moved reference maximum
-  auto softmax = [&]() {
-    float mx = sacc[0][0];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
-    mx = half_max(mx) * p.scale_log2;
-    if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-    }
-    const float mc = (m_run == -INFINITY) ? 0.f : m_run;
-    float ls = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = fast_exp2(__builtin_fmaf(sacc[kb][r], p.scale_log2, -mc));
-        ls += e;
-        sacc[kb][r] = e;
-      }
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        X8 pk;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pk[j] = E::from_float(sacc[kb][8 * t2 + j]);
-        pf[kb][t2] = pk;
-      }
-    }
-    l_run += ls;
-  };
-  // O^T += V(t)^T P^T(t)
-  auto pv = [&](int t) {
-    MSD_LDS const char* vb_base = smem + (2 + (t & 1)) * kTileBytes;
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          MSD_LDS const char* src = vb_base + (kb * 32 + 16 * t2) * kRowBytes + v_row_off + ((db ^ v_swz) << 6);
-          const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)src);
-          const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MSD_LDS s16x4_t*)(src + 8 * kRowBytes));
-          union { s16x4_t s[2]; X8 x; } u;
-          u.s[0] = lo;
-          u.s[1] = hi;
-          oacc[db] = E::mfma32(u.x, pf[kb][t2], oacc[db]);
-        }
-  };
-
-  // ---- prologue: K(0), V(0), K(1) in LDS; S(0) for everybody, P(0) for the early waves ----------------
-  load_k(0);
-  load_v(0);
-  if (n_tiles > 1) load_k(1);
-  __builtin_amdgcn_s_waitcnt(0x0f70);
-  __syncthreads();
-  qk(0);
-  if (!late) softmax();
-
-  for (int t = 0; t < n_tiles; ++t) {
-    // interval t: V(t) and K(t+1) are in LDS; fetch V(t+1) and K(t+2) for the next interval
-    if (t + 1 < n_tiles) load_v(t + 1);
-    if (t + 2 < n_tiles) load_k(t + 2);
-    if (late) softmax();
-    pv(t);
-    if (t + 1 < n_tiles) {
-      qk(t + 1);
-      if (!late) softmax();
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-  }
-
-  // ---- epilogue ---------------------------------------------------------------------------------------
-  MSD_LDS char* ost = smem + wave * 32 * kORowBytes;
-  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
-  const float l_tot = half_sum(l_run);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  const int qrow_l = q0 + wave * 32 + l32;
-  if (p.lse && h == 0 && qrow_l < p.Sq) {
-    const long long li = ((long long)b * p.N + n) * p.Sq + qrow_l;
-    p.lse[li] = l_tot > 0.f ? m_run * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
-  }
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      typename E::x4 pk;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pk[j] = E::from_float(oacc[db][4 * g + j] * inv);
-      const int d = db * 32 + 8 * g + 4 * h;
-      *(MSD_LDS typename E::x4*)(ost + l32 * kORowBytes + d * 2) = pk;
-    }
-  __builtin_amdgcn_wave_barrier();
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int c = i * 64 + lane;
-    const int row = c >> 4, c16 = c & 15;
-    const int qrow = q0 + wave * 32 + row;
-    const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16);
-    const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16 + 8);
-    if (qrow < p.Sq) *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
-  }
-#endif
-}
-
-template <int DT>
-static int launch_fa_pp(const FaParams& p, hipStream_t stream) {
-  constexpr int kLds = 4 * 128 * 256;  // K0 K1 V0 V1
-  auto kern = fa_fwd_pp_kernel<DT>;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-    return MSD_ERR_LAUNCH;
-  const int total = p.B * p.N * ((p.Sq + 255) / 256);
-  hipLaunchKernelGGL(kern, dim3((total + 7) / 8 * 8), dim3(512), kLds, stream, p);
-  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
-}
-
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -928,7 +673,6 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   p.map_mode = g_map_mode;
   if (dtype == MSD_DTYPE_BF16) {
     switch (g_dense_variant) {
-      case 4: return launch_fa_pp<MSD_DTYPE_BF16>(p, stream);
       case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);
       case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
       case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);
