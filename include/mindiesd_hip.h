@@ -89,6 +89,27 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
                                         float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
                                         const int* order, hipStream_t stream);
 
+/* The same with the query side addressed through a table (self-attention, S tokens): query position i - the
+ * position that the block lists and the rows of k and v refer to - is row token_order[i] of q and of out
+ * (every row exactly once).  With the table of mindiesd_rf_token_order, k and v permuted by
+ * mindiesd_rf_rearrange_pool and q, out in their original order, this is attention on
+ * rearrange_with_remaining(q) followed by inv_rearrange_with_remaining of the result
+ * (mindiesd/layers/flash_attn/sparse_flash_attn_rf_v2.py:137-289, sparse_flash_attn_rf_v3.py:22-97, 248-295)
+ * without the permuted copy of q and without the inverse pass. */
+int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                               int dtype, int B, int N, int Nkv, int S, int D,
+                                               long long q_sb, long long q_sn, long long q_ss,
+                                               long long k_sb, long long k_sn, long long k_ss,
+                                               long long v_sb, long long v_sn, long long v_ss,
+                                               long long o_sb, long long o_sn, long long o_ss,
+                                               float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                               const int* token_order, hipStream_t stream);
+
+/* token_order[i] (int32, S entries) = row of the original [text | image (t,h,w)] sequence that holds the
+ * token at position i of RainFusion's [image in 8x8-window order | text] sequence (the index map behind
+ * rearrange_with_remaining, sparse_flash_attn_rf_v2.py:137-196, 297-312). */
+int mindiesd_rf_token_order(int* token_order, int S, int t, int h, int w, int txt_len, hipStream_t stream);
+
 /* ---- adaptive block-sparse attention (mask estimate + attention) ------------------------------------------
  * Block-sparse attention as above (queries and keys of equal length S) with an optional causal mask inside
  * the selected blocks: key j is visible to query i iff j <= i.  Replaces aclnnAdaBlockSparseAttention behind

@@ -47,6 +47,7 @@ struct FaParams {
   int kb_stride;
   int QB;
   const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
+  const int* tok;    // GATHER instantiations: [Sq] row of q/out that holds the token at query position i
   int map_mode;      // 0: consecutive query tiles of a head share an XCD; 1: linear block order
   // general mode (MODE = 1 instantiations only)
   const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
@@ -102,7 +103,11 @@ __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu
 
 // Register budget: 8 wavefronts per CU (two per SIMD) in every configuration, i.e. at most 256
 // registers per lane; the 4-wave configurations run two workgroups per CU.
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0>
+// GATHER: the query sequence the kernel works on is a permutation of the rows of q and out (p.tok): query rows
+// are fetched and output rows stored through the table.  K and V stay contiguous in the permuted order: tiles
+// gathered row by row through the same table measured 8 % slower (the block-sparse walk is bound by the L2-miss
+// path, and 2 KiB runs use it worse than 32 KiB tiles), more than the permuted copies of K and V cost.
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -167,7 +172,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   for (int qb = 0; qb < C::kNQB; ++qb) {
     const int qrow = q0 + wave * QPW + qb * 32 + l32;
     const bool ok = qrow < Sq;
-    const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * h;
+    const int qsrc = GATHER ? p.tok[ok ? qrow : 0] : (ok ? qrow : 0);
+    const T* src = qg + (long long)qsrc * p.q_ss + 8 * h;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       X8 v = *(const X8*)(src + 16 * ks);
@@ -542,7 +548,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int qrow_l = q0 + wave * QPW + qb * 32 + l32;
     if (p.lse && h == 0 && qrow_l < Sq) {
-      const long long li = ((long long)b * p.N + n) * p.Sq + qrow_l;
+      const long long li = ((long long)b * p.N + n) * p.Sq + (GATHER ? p.tok[qrow_l] : qrow_l);
       p.lse[li] = l_tot > 0.f ? m_run[qb] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
     }
 #pragma unroll
@@ -566,7 +572,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * C::kORowBytes + c16 * 16 + 8);
       if (qrow < Sq) {
         i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
-        *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = v;
+        const int orow = GATHER ? p.tok[qrow] : qrow;
+        *(i32x4_t*)(og + (long long)orow * p.o_ss + c16 * 8) = v;
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -574,10 +581,10 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
-  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE>;
+  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE, GATHER>;
   // per device and idempotent, so it is simply repeated on every launch
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
     return MSD_ERR_LAUNCH;
@@ -659,6 +666,29 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
   // one query block per workgroup, 64-key sub-tiles, two workgroups per CU
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
+}
+
+// The same with the query side addressed through a table: query position i (the position the block lists and the
+// rows of k and v refer to) is row token_order[i] of q and of out (S entries, every row exactly once).  With k and
+// v permuted and q, out left in their original order this saves the permuted copy of q and the inverse
+// permutation of the output.
+int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                               int dtype, int B, int N, int Nkv, int S, int D, long long q_sb,
+                                               long long q_sn, long long q_ss, long long k_sb, long long k_sn,
+                                               long long k_ss, long long v_sb, long long v_sn, long long v_ss,
+                                               long long o_sb, long long o_sn, long long o_ss, float scale,
+                                               const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                               const int* token_order, hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, S, S, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (!blk_idx || !blk_cnt || kb_stride <= 0 || !token_order) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, S, S, st, scale);
+  p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.tok = token_order;
+  p.map_mode = g_map_mode;
+  p.QB = (S + 127) / 128;
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, true>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, true>(p, stream);
 }
 
 int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,

@@ -290,6 +290,15 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
 #endif
 }
 
+// tok[i] = row of the original [text | image] sequence that holds the token at position i of the permuted
+// [image in window order | text] sequence: the table the gather mode of the attention kernel reads.
+__global__ __launch_bounds__(256) void rf_token_order_kernel(int* tok, int S, int txt_len, Grid3 g) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= S) return;
+  const int s_img = S - txt_len;
+  tok[i] = i < s_img ? txt_len + window_source(i, g) : i - s_img;
+}
+
 // int8 mask rows -> ascending index lists + counts (used when a caller supplies the mask).
 __global__ __launch_bounds__(256) void mask_to_index_kernel(const signed char* mask, int* blk_idx, int* blk_cnt,
                                                             int QB, int KB, int kb_stride) {
@@ -377,6 +386,14 @@ int mindiesd_rf_rearrange_pool(const void* q, const void* k, const void* v, void
     hipLaunchKernelGGL(rf_rearrange_pool_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, p);
   else
     hipLaunchKernelGGL(rf_rearrange_pool_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+int mindiesd_rf_token_order(int* token_order, int S, int t, int h, int w, int txt_len, hipStream_t stream) {
+  if (!token_order || S <= 0 || txt_len < 0 || t <= 0 || h < 8 || w < 8) return MSD_ERR_BAD_ARG;
+  if ((long long)t * h * w + txt_len != S) return MSD_ERR_BAD_ARG;
+  hipLaunchKernelGGL(rf_token_order_kernel, dim3((S + 255) / 256), dim3(256), 0, stream, token_order, S, txt_len,
+                     Grid3{t, h, w});
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 

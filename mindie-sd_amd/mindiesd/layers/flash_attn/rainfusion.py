@@ -55,7 +55,7 @@ def _run_rearrange(srcs, dsts, pool, layout, grid, txt_len, inverse):
     x = srcs[0]
     b, n, s = _dims(x, layout)
     ptr = lambda lst, i: lst[i].data_ptr() if i < len(lst) and lst[i] is not None else None
-    d0 = dsts[0] if dsts and dsts[0] is not None else x
+    d0 = next((d for d in (dsts or []) if d is not None), x)  # all destinations share one set of strides
     if pool is not None:
         psb, psn, psblk = _pool_strides(pool, layout)
         pst = b * pool.stride(0)
@@ -252,10 +252,40 @@ def get_blockwise_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_sha
 # ------------------------------------------------------------------------------------------------
 # block-sparse attention kernels (rf_v2.py:351-381, rf_v3.py:122-190)
 # ------------------------------------------------------------------------------------------------
-def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, layout="BNSD", return_lse=False):
+_token_order_cache = {}
+
+
+def token_order(latent_shape, txt_len, device):
+    """int32 [t*h*w + txt_len]: row of the original [text | image] sequence that holds the token at position i
+    of RainFusion's [image in 8x8-window order | text] sequence (the index map of rearrange_with_remaining,
+    rf_v2.py:137-196, 297-312).  Built once per (grid, text length, device)."""
+    t, h, w = (int(v) for v in latent_shape)
+    if t <= 0 or h < 8 or w < 8:
+        raise ParametersInvalid(f"latent_shape_q must be (t, h, w) with h >= 8 and w >= 8, but got {latent_shape}.")
+    dev = torch.device(device)
+    key = (t, h, w, int(txt_len), dev.type, dev.index if dev.index is not None else torch.cuda.current_device())
+    tok = _token_order_cache.get(key)
+    if tok is None:
+        s = t * h * w + int(txt_len)
+        tok = torch.empty((s,), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _native.lib().mindiesd_rf_token_order(tok.data_ptr(), s, t, h, w, int(txt_len), _native.stream_ptr(dev))
+        _native.check(rc, "mindiesd_rf_token_order")
+        if len(_token_order_cache) >= 16:
+            _token_order_cache.clear()
+        _token_order_cache[key] = tok
+    return tok
+
+
+def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, layout="BNSD", return_lse=False,
+                                 order=None):
     """Attention of every 128-row query block over the key blocks listed for it.
     ``blk_idx`` int32 [B, N, qb, stride] ascending block ids, ``blk_cnt`` int32 [B, N, qb].
-    A query block with an empty list yields zeros."""
+    A query block with an empty list yields zeros.
+    ``order`` (int32 [S], from :func:`token_order`): query position i - the position the lists and the rows of
+    key and value refer to - is row ``order[i]`` of query and of the output (self-attention only): with key and
+    value permuted and query left as it is, this is attention on the permuted query and the inverse permutation
+    of the result in one pass."""
     for name, t in (("query", query), ("key", key), ("value", value)):
         _check_gpu16(t, name)
     q, k, v = _aligned(query), _aligned(key), _aligned(value)
@@ -269,6 +299,20 @@ def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, lay
         raise ParametersInvalid(f"block lists must be contiguous int32 [B,N,{qb},stride] / [B,N,{qb}].")
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     lse = torch.empty((b, n, sq), dtype=torch.float32, device=q.device) if return_lse else None
+    if order is not None:
+        if (order.dtype != torch.int32 or order.dim() != 1 or order.shape[0] != sq or skv != sq or not order.is_contiguous()
+                or order.device != q.device):
+            raise ParametersInvalid(f"order must be a contiguous int32 [{sq}] tensor on the inputs' device "
+                                    "(self-attention only).")
+        with torch.cuda.device(q.device):
+            rc = _native.lib().mindiesd_block_sparse_attention_gather_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
+                _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, q.shape[-1],
+                *_strides_bns(q, layout), *_strides_bns(k, layout), *_strides_bns(v, layout), *_strides_bns(out, layout),
+                float(scale), blk_idx.data_ptr(), blk_cnt.data_ptr(), blk_idx.shape[3], order.data_ptr(),
+                _native.stream_ptr(q.device))
+        _native.check(rc, "mindiesd_block_sparse_attention_gather_fwd")
+        return (out, lse) if return_lse else out
     with torch.cuda.device(q.device):
         rc = _native.lib().mindiesd_block_sparse_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
@@ -336,14 +380,33 @@ def bsa_sparse_attention_v3(q, k, v, latent_shape_q, latent_shape_k=None, txt_le
         scale = float(q.shape[-1]) ** -0.5
     if pool_size != BLOCK:
         raise ParametersInvalid(f"pool_size only supports {BLOCK}, but got {pool_size}.")
+    # Only key and value are copied into the window order (their tiles must be contiguous for the kernel's
+    # LDS-DMA); the query is pooled through the order and read by the attention kernel through the same table,
+    # which also stores the output rows straight to their original places.
+    _check_layout(input_layout)
+    for name, t in (("query", q), ("key", k), ("value", v)):
+        _check_gpu16(t, name)
+    if not (q.shape == k.shape == v.shape and q.dtype == k.dtype == v.dtype):
+        raise ParametersInvalid("RainFusion needs query, key and value of one shape and dtype "
+                                "(self-attention over the latent grid).")
+    q, k, v = _aligned(q), _aligned(k), _aligned(v)
+    if not _same_strides((q, k, v)):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    b, n, s = _dims(q, input_layout)
+    grid = _check_grid(latent_shape_q, s - txt_len)
+    k_ = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    v_ = torch.empty(v.shape, dtype=v.dtype, device=v.device)
     if cached_mask is None:
-        q_, k_, v_, pool = _rearrange_qkv(q, k, v, txt_len, latent_shape_q, input_layout, True)
+        nb = (s - txt_len + BLOCK - 1) // BLOCK + (txt_len + BLOCK - 1) // BLOCK
+        shape = (3 * b, n, nb, q.shape[-1]) if input_layout == "BNSD" else (3 * b, nb, n, q.shape[-1])
+        pool = torch.empty(shape, dtype=q.dtype, device=q.device)
+        _run_rearrange([q, k, v], [None, k_, v_], pool, input_layout, grid, txt_len, 0)
         new_mask, idx, cnt, _, _ = _block_mask(pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout,
                                                protect_first_frame, keep_diagonal, True, True, False)
     else:
-        q_, k_, v_, _ = _rearrange_qkv(q, k, v, txt_len, latent_shape_q, input_layout, False)
+        _run_rearrange([k, v], [k_, v_], None, input_layout, grid, txt_len, 0)
         new_mask = cached_mask
         idx, cnt = mask_to_lists(cached_mask)
-    out = block_sparse_attention_lists(q_, k_, v_, idx, cnt, scale, input_layout)
-    out = do_tensor_inv_rearrange(out, txt_len, latent_shape_q, latent_shape_k, input_layout)
+    out = block_sparse_attention_lists(q, k_, v_, idx, cnt, scale, input_layout,
+                                       order=token_order(grid, txt_len, q.device))
     return out, new_mask

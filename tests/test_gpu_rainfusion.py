@@ -200,6 +200,29 @@ def test_rf_v3_end_to_end_vs_oracle(cuda, grid, layout):
     assert mask2 is mask and torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("layout", ["BNSD", "BSND"])
+@pytest.mark.parametrize("grid,txt", [("div", 0), ("nodiv_both", 0), ("nodiv_h", 256), ("nodiv_w", 128)])
+def test_fused_permutation_equals_explicit_passes(cuda, grid, txt, layout):
+    """The end-to-end call reads q, k, v and writes the output through the window-order table; the explicit
+    chain permute+pool -> mask -> attention -> inverse permute (the reference's sequence of calls,
+    rf_v3.py:248-295) must give the same mask and bit-identical output."""
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    g3 = GRIDS[grid]
+    q, k, v = (t.to(cuda) for t in _structured_qkv(layout, 2, g3, txt, seed=77))
+    tok = rf.token_order(g3, txt, cuda)
+    want_tok = torch.cat([torch.as_tensor(orf.window_order(*g3)) + txt, torch.arange(txt)]).to(torch.int32)
+    assert torch.equal(tok.cpu(), want_tok)
+    out, mask = rf.bsa_sparse_attention_v3(q, k, v, g3, txt_len=txt, sparsity=0.7, input_layout=layout,
+                                           keep_diagonal=True)
+    q_, k_, v_, pool = rf.do_tensor_rearrange_pooling(q, k, v, txt, 128, g3, g3, layout)
+    mask_x = rf.get_blockwise_mask(pool, txt, 0.7, 128 ** -0.5, 128, g3, g3, layout, return_binary=True,
+                                   keep_diagonal=True)
+    out_x = rf.rain_fusion_attention_v3(q_, k_, v_, mask_x, input_layout=layout)
+    out_x = rf.do_tensor_inv_rearrange(out_x, txt, g3, g3, layout)
+    assert torch.equal(mask, mask_x)
+    assert torch.equal(out, out_x)
+
+
 def test_rf_v2_equals_rf_v3(cuda):
     import mindiesd
     g3 = GRIDS["nodiv_w"]
