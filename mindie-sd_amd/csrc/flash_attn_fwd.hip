@@ -88,15 +88,19 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // LDS-DMA of one K tile and one V tile: every wave issues G pairs of 1 KiB transfers.
+// Group i of a wave lies 4 * NWAVES rows below group 0 (a multiple of 16, so the swizzles are the same): one
+// per-lane offset per operand serves all groups, the rest goes into the scalar offset.
 template <int G, int NWAVES>
 __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu_buffer_rsrc_t v_rsrc,
-                                         MSD_LDS char* kb, MSD_LDS char* vb, const int (&k_voff)[G],
-                                         const int (&v_voff)[G], int wave, int k_soff, int v_soff) {
+                                         MSD_LDS char* kb, MSD_LDS char* vb, int k_voff, int v_voff, int wave,
+                                         int k_soff, int v_soff, int k_row_bytes, int v_row_bytes) {
 #pragma unroll
   for (int i = 0; i < G; ++i) {
     const int g = i * NWAVES + wave;  // 4-row group of the tile
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g * 1024), 16, k_voff[i], k_soff, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g * 1024), 16, v_voff[i], v_soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g * 1024), 16, k_voff,
+                                             k_soff + i * 4 * NWAVES * k_row_bytes, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g * 1024), 16, v_voff,
+                                             v_soff + i * 4 * NWAVES * v_row_bytes, 0, 0);
   }
 }
 #endif
@@ -216,18 +220,18 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)vg, 0, Skv > 0 ? (int)(((long long)(Skv - 1) * p.v_ss + C::kD) * 2) : 0, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
-  int k_voff[C::kGroupsPerWave], v_voff[C::kGroupsPerWave];
-#pragma unroll
-  for (int i = 0; i < C::kGroupsPerWave; ++i) {
-    const int row = 4 * (i * NWAVES + wave) + (lane >> 4);
+  static_assert((4 * NWAVES) % 16 == 0, "groups of one wave must share their swizzle");
+  int k_voff, v_voff;
+  {
+    const int row = 4 * wave + (lane >> 4);
     const int pc = lane & 15;
-    k_voff[i] = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
-    v_voff[i] = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
+    k_voff = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
+    v_voff = row * v_row_bytes + ((pc ^ ((row & 3) << 2)) << 4);
   }
   auto load_tile = [&](int key0, int stage) {
     MSD_LDS char* kb = smem + stage * C::kStageBytes;
     tile_dma<C::kGroupsPerWave, NWAVES>(k_rsrc, v_rsrc, kb, kb + C::kTileBytes, k_voff, v_voff, wave,
-                                        key0 * k_row_bytes, key0 * v_row_bytes);
+                                        key0 * k_row_bytes, key0 * v_row_bytes, k_row_bytes, v_row_bytes);
   };
 
   // per-lane constant parts of the LDS read addresses
