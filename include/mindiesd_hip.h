@@ -134,11 +134,16 @@ int mindiesd_ada_block_sparse_attention_fwd(const void* q, const void* k, const 
  * mindiesd_sbe_select: per row, key blocks in descending score order (the last block left out) are kept
  *   until their running sum reaches threshold * total, at most row_sparse * NB of them; the first block is
  *   kept if keep_sink, the last if keep_recent.  mask int8 [BN][NB][pitch] (pitch >= NB, zero padded; the
- *   reference uses pitch = NB rounded up to 32), count int32 [BN][NB]. */
+ *   reference uses pitch = NB rounded up to 32), count int32 [BN][NB].
+ * causal != 0 (test_sparseblockestimate.py:71-78, 121-127): the block rows of one step of 1024 query tokens see
+ *   the strided columns below min(col_cap, 128 * (step + 1)) with col_cap = S / 8; row i of the selection ranks
+ *   its first i + 1 blocks with the diagonal block in the place of the last one, rows 0 and 1 keep their whole
+ *   prefix, blocks above the diagonal are never selected. */
 int mindiesd_sbe_block_scores(const void* pmat, float* scores, int dtype, int BN, int Sr, int ldp, float scale,
-                              hipStream_t stream);
+                              int causal, int col_cap, hipStream_t stream);
 int mindiesd_sbe_select(const float* scores, signed char* mask, int* count, int BN, int NB, int pitch,
-                        float threshold, float row_sparse, int keep_sink, int keep_recent, hipStream_t stream);
+                        float threshold, float row_sparse, int keep_sink, int keep_recent, int causal,
+                        hipStream_t stream);
 
 /* ---- RainFusion2.0 mask pipeline ---------------------------------------------------------------------
  * Token permutation into 8x8 spatial windows (+ optional block mean pooling) of up to three tensors

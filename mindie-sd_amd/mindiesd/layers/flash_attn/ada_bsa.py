@@ -42,8 +42,6 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
     if stride != STRIDE or sparse_size != BLOCK:
         raise RuntimeError(f"sparse_block_estimate supports stride {STRIDE} and sparse_size {BLOCK} only, "
                            f"got {stride} and {sparse_size}")
-    if causal:
-        raise RuntimeError("sparse_block_estimate: causal estimation is not available in this build")
     s_tokens = query.shape[2] if input_layout == "BNSD" else query.shape[1]
     if s_tokens > MAX_ESTIMATE_TOKENS:
         raise RuntimeError(f"sparse_block_estimate: sequences longer than {MAX_ESTIMATE_TOKENS} tokens are switched off in "
@@ -75,14 +73,15 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
             g1 = min(b * n, g0 + group)
             pmat = torch.bmm(qp[g0:g1], kp[g0:g1].transpose(1, 2))  # [g, sr, ldp] raw strided products
             rc = lib.mindiesd_sbe_block_scores(pmat.data_ptr(), scores[g0:g1].data_ptr(), _native.DTYPE_CODE[q.dtype],
-                                               g1 - g0, sr, ldp, float(scale_value), _native.stream_ptr(q.device))
+                                               g1 - g0, sr, ldp, float(scale_value), int(bool(causal)),
+                                               max(1, s // STRIDE), _native.stream_ptr(q.device))
             _native.check(rc, "mindiesd_sbe_block_scores")
             del pmat
         mask = torch.empty((b, n, nb, pitch), dtype=torch.int8, device=q.device)
         count = torch.empty((b, n, nb), dtype=torch.int32, device=q.device)
         rc = lib.mindiesd_sbe_select(scores.data_ptr(), mask.data_ptr(), count.data_ptr(), b * n, nb, pitch,
                                      float(threshold), float(row_sparse), int(bool(keep_sink)), int(bool(keep_recent)),
-                                     _native.stream_ptr(q.device))
+                                     int(bool(causal)), _native.stream_ptr(q.device))
         _native.check(rc, "mindiesd_sbe_select")
     if return_scores:
         return mask, count, scores.view(b, n, nb, nb)

@@ -3,10 +3,10 @@
 Restates the numpy statements the reference's tests hold for its two in-tree AscendC kernels:
 ``sparse_estimate`` follows tests/plugin/test_sparseblockestimate.py:24-36 (softmax_flash) and :49-145
 (sparse_estimate_cpu), ``ada_block_sparse_attention`` follows
-tests/plugin/test_adablocksparseattention.py:35-87.  The estimate is restated for the non-causal case
-(the only one the reference's test exercises, test_sparseblockestimate.py:166); the reference's own
-tolerance for it is a mask difference below 2 % of the selected blocks and fewer than 1 % omitted blocks
-(:231-241).
+tests/plugin/test_adablocksparseattention.py:35-87.  The reference's test exercises the non-causal estimate only
+(test_sparseblockestimate.py:166); the causal branches of its numpy statement are restated as they stand.  Its
+own tolerance for the estimate is a mask difference below 2 % of the selected blocks and fewer than 1 % omitted
+blocks (:231-241).
 """
 import numpy as np
 import torch
@@ -39,19 +39,23 @@ def strided_scores(q, k, stride=8):
     return np.dot(qs / (np.sqrt(d) * stride), ks.T)
 
 
-def block_scores(q, k, blocksize=128, stride=8):
+def block_scores(q, k, blocksize=128, stride=8, causal=False):
     """Share of the estimated attention mass per (query block, key block), with the reference's loop
     structure: 128 strided rows at a time, columns in steps of 1024 with a running softmax, first reduction
     over groups of blocksize/stride columns, rescaling to the final maximum and sum, second reduction over
-    groups of rows (:58-119)."""
+    groups of rows (:58-119).  ``causal``: a step of 1024 query tokens sees the keys up to its own end, cut
+    down to whole groups of ``stride`` tokens (:71, :78); the result then has a row of blocks per query
+    block but only as many columns as the last step saw, earlier rows are zero padded."""
     reduce_size = blocksize // stride
     seq = q.shape[0]
+    nb = (seq + blocksize - 1) // blocksize
     out = []
     for r0 in range(0, seq, M_ROWS * stride):
         qc = q[r0:r0 + M_ROWS * stride]
+        kseq = seq if not causal else (r0 + qc.shape[0]) // stride * stride
         first, maxes, x_max, x_sum = [], [], None, None
-        for c0 in range(0, seq, N_COLS * stride):
-            p = strided_scores(qc, k[c0:c0 + N_COLS * stride], stride)
+        for c0 in range(0, kseq, N_COLS * stride):
+            p = strided_scores(qc, k[c0:min(kseq, c0 + N_COLS * stride)], stride)
             p, x_max, x_sum = softmax_flash(p, x_max, x_sum)
             pc = p.shape[1] % reduce_size
             if pc:
@@ -62,7 +66,10 @@ def block_scores(q, k, blocksize=128, stride=8):
         for part, mx in zip(first, maxes):
             part = _pad_rows(part * (np.exp(mx - x_max) / x_sum), reduce_size)
             rows.append(part.reshape(-1, reduce_size, part.shape[1]).sum(axis=1))
-        out.append(np.concatenate(rows, axis=-1))
+        blk = np.concatenate(rows, axis=-1)
+        if blk.shape[1] < nb:
+            blk = np.concatenate([blk, np.zeros((blk.shape[0], nb - blk.shape[1]), dtype=blk.dtype)], axis=1)
+        out.append(blk[:, :max(nb, blk.shape[1])])
     return np.concatenate(out, axis=0)
 
 
@@ -88,8 +95,11 @@ def select_blocks(score_row, threshold, force_sparse, keep_sink=True, keep_recen
 
 
 def sparse_estimate(query, key, blocksize=128, stride=8, threshold=0.5, force_sparse=1.0, keep_sink=True,
-                    keep_recent=True):
-    """[B, N, S, D] query / key (any float dtype) -> boolean mask [B, N, nb, nb], nb = ceil(S / blocksize)."""
+                    keep_recent=True, causal=False):
+    """[B, N, S, D] query / key (any float dtype) -> boolean mask [B, N, nb, nb], nb = ceil(S / blocksize).
+    ``causal`` (:121-127, :140): row i selects among its first i + 1 blocks, the diagonal block standing where
+    the last block stands otherwise (forced only with ``keep_recent``, the kernel's setDiag,
+    sparse_block_estimate.h:1047-1049); rows 0 and 1 keep their whole prefix."""
     bs, nq, seq, _ = query.shape
     gqa = nq // key.shape[1]
     nb = (seq + blocksize - 1) // blocksize
@@ -97,9 +107,15 @@ def sparse_estimate(query, key, blocksize=128, stride=8, threshold=0.5, force_sp
     qf, kf = query.float().numpy(), key.float().numpy()
     for bi in range(bs):
         for ni in range(nq):
-            sc = block_scores(qf[bi, ni], kf[bi, ni // gqa], blocksize, stride)
+            sc = block_scores(qf[bi, ni], kf[bi, ni // gqa], blocksize, stride, causal)
             for i in range(nb):
-                mask[bi, ni, i] = select_blocks(sc[i, :nb], threshold, force_sparse, keep_sink, keep_recent)
+                if not causal:
+                    mask[bi, ni, i] = select_blocks(sc[i, :nb], threshold, force_sparse, keep_sink, keep_recent)
+                elif i <= 1:
+                    mask[bi, ni, i, :i + 1] = True
+                else:
+                    mask[bi, ni, i, :i + 1] = select_blocks(sc[i, :i + 1], threshold, force_sparse, keep_sink,
+                                                            keep_recent)
     return mask
 
 

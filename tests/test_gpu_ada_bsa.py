@@ -48,6 +48,35 @@ def test_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, dtype):
         assert (got[0, h] < want[0, h]).sum() / selected < 0.01
 
 
+@pytest.mark.parametrize("keep_recent", [True, False])
+@pytest.mark.parametrize("s,threshold,row_sparse", [(2048, 0.85, 1.0), (3000, 0.6, 0.5), (1031, 0.9, 1.0)])
+def test_causal_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, keep_recent):
+    """Causal estimate: keys limited per step of 1024 query tokens, selection inside the lower triangle."""
+    import mindiesd  # noqa: F401
+    from mindiesd.layers.flash_attn.ada_bsa import sparse_block_estimate
+    q, k = _structured((1, 2, s, 128), 11, torch.float16), _structured((1, 2, s, 128), 13, torch.float16)
+    scale = 128 ** -0.5 / 8
+    smask, sct, scores = sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=scale, threshold=threshold,
+                                               causal=True, keep_recent=keep_recent, row_sparse=row_sparse,
+                                               return_scores=True)
+    nb = (s + 127) // 128
+    got = smask.cpu().numpy().astype(bool)[..., :nb]
+    assert np.array_equal(sct.cpu().numpy(), got.sum(-1))
+    assert not np.triu(got[0, 0], 1).any() and not np.triu(got[0, 1], 1).any()
+    assert got[0, :, 0, 0].all() and got[0, :, 1, :2].all()
+    want_sc = oab.block_scores(q[0, 0].float().numpy(), k[0, 0].float().numpy(), causal=True)
+    got_sc = scores.cpu().numpy()[0, 0]
+    assert np.abs(np.tril(got_sc) - np.tril(want_sc[:nb, :nb])).max() < 2e-2
+    want = oab.sparse_estimate(q, k, threshold=threshold, force_sparse=row_sparse, keep_recent=keep_recent,
+                               causal=True)
+    for h in range(2):
+        selected = want[0, h].sum()
+        assert (got[0, h] != want[0, h]).sum() / selected < 0.02
+        assert (got[0, h] < want[0, h]).sum() / selected < 0.01
+    if keep_recent:
+        assert np.diag(got[0, 0]).all()
+
+
 def test_block_scores_and_selection_separately(cuda):
     from mindiesd.layers.flash_attn.ada_bsa import sparse_block_estimate
     s = 2500
@@ -130,8 +159,6 @@ def test_ada_bsa_errors(cuda):
         torch.ops.mindiesd.sparse_block_estimate(q, q, input_layout="TND", causal=False)
     with pytest.raises(RuntimeError):
         torch.ops.mindiesd.sparse_block_estimate(q, q, stride=4, causal=False)
-    with pytest.raises(RuntimeError):
-        torch.ops.mindiesd.sparse_block_estimate(q, q, causal=True)
     big = torch.zeros(1, 1, 3073, 128, dtype=torch.float16, device=cuda)
     with pytest.raises(RuntimeError, match="switched off"):
         torch.ops.mindiesd.sparse_block_estimate(big, big, causal=False)

@@ -86,3 +86,44 @@ def test_ada_attention_reduces_to_dense_and_causal():
     m[0, 1, 2] = False
     out = oab.ada_block_sparse_attention(q, k[:, :1], v[:, :1], m, blocksize=128)
     assert not out[0, 1, 256:].any() and out[0, 0].abs().sum() > 0
+
+
+# ---- causal estimate (restated from the branches of the reference's numpy statement that its test does not run) ----
+def _qk(s, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(1, 1, s, 128, generator=g), torch.randn(1, 1, s, 128, generator=g)
+
+
+def test_causal_estimate_stays_in_the_lower_triangle_and_keeps_first_rows():
+    q, k = _qk(2100, 1)
+    m = oab.sparse_estimate(q, k, threshold=0.6, force_sparse=0.5, causal=True)[0, 0]
+    assert not np.triu(m, 1).any()
+    assert m[0, 0] and m[1, :2].all()
+    assert m[:, 0].all() and np.diag(m).all()          # sink and diagonal forced
+    m2 = oab.sparse_estimate(q, k, threshold=0.6, force_sparse=0.5, causal=True, keep_recent=False)[0, 0]
+    assert not np.diag(m2)[2:].any()                   # the diagonal block is ranked as zero and not forced
+
+
+def test_causal_estimate_with_threshold_one_is_the_lower_triangle():
+    q, k = _qk(1500, 2)
+    m = oab.sparse_estimate(q, k, threshold=1.0, force_sparse=1.0, causal=True)[0, 0]
+    assert np.array_equal(m, np.tril(np.ones_like(m)))
+
+
+def test_causal_scores_ignore_keys_after_the_query_step():
+    """A step of 1024 query tokens sees the keys up to its own end: later keys change nothing in its rows."""
+    q, k = _qk(2048 + 512, 3)
+    a = oab.block_scores(q[0, 0].numpy(), k[0, 0].numpy(), causal=True)
+    k2 = k.clone()
+    k2[0, 0, 1024:] += 3.0
+    b = oab.block_scores(q[0, 0].numpy(), k2[0, 0].numpy(), causal=True)
+    assert np.array_equal(a[:8], b[:8]) and not np.allclose(a[8:16], b[8:16])
+    assert not a[:8, 8:].any() and not a[8:16, 16:].any()
+    np.testing.assert_allclose(a[:8].sum(1), 16.0, rtol=1e-4)      # 16 strided rows of unit mass per block row
+
+
+def test_causal_scores_of_a_single_step_equal_the_plain_ones():
+    q, k = _qk(1024, 4)
+    a = oab.block_scores(q[0, 0].numpy(), k[0, 0].numpy(), causal=True)
+    b = oab.block_scores(q[0, 0].numpy(), k[0, 0].numpy(), causal=False)
+    assert np.array_equal(a, b)
