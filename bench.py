@@ -252,6 +252,7 @@ def extra_fp8(device, steps, warmup):
     q, k, v = outlier_inputs(cfg, device, seed=4)
     scale = cfg["D"] ** -0.5
     bf16_ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)
+    # default recipe: block scales amax/448, as the reference's block quantisation leaves them
     e2e_ms, _ = time_steps(lambda: f8.fp8_attention_forward(q, k, v), steps, warmup)
     quant = lambda: (_block_quant(q, 128, "BNSD"), _block_quant(k, 128, "BNSD"), f8.quantize_v_per_channel(v))
     (q8, qs), (k8, ks), (v8t, vs) = quant()
@@ -260,6 +261,16 @@ def extra_fp8(device, steps, warmup):
     out8 = f8.fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale)
     out16 = mindiesd.attention_forward(q, k, v, head_first=True)
     cos = float(torch.nn.functional.cosine_similarity(out8.float().flatten(), out16.float().flatten(), dim=0))
+    del q8, k8, out8
+    # the optional recipe: power-of-two block scales, softmax scale folded into the query (log2-domain kernel)
+    pre = scale * f8.LOG2E
+    (a8, asq), (b8, bsk) = _block_quant(q, 128, "BNSD", pre, True), _block_quant(k, 128, "BNSD", 1.0, True)
+    pkern_ms, _ = time_steps(lambda: f8.fp8_attention_quantized(a8, asq, b8, bsk, v8t, vs, scale, log2_domain=True),
+                             steps, warmup)
+    pe2e_ms, _ = time_steps(lambda: f8.fp8_attention_forward(q, k, v, recipe="pow2"), steps, warmup)
+    outp = f8.fp8_attention_quantized(a8, asq, b8, bsk, v8t, vs, scale, log2_domain=True)
+    cos_p = float(torch.nn.functional.cosine_similarity(outp.float().flatten(), out16.float().flatten(), dim=0))
+    del a8, b8, outp
     # the FP8RotateQuantFA recipe: an orthogonal (Hadamard) rotation of q and k spreads the outliers over the
     # channels before quantisation; here it runs inside the quantisation pass
     from mindiesd.layers.quant.block_quant import _rot_block_quant
@@ -273,21 +284,30 @@ def extra_fp8(device, steps, warmup):
                                    _block_quant(torch.matmul(k, rot), 128, "BNSD")), steps, warmup)
     out8r = f8.fp8_attention_forward(q, k, v, q_rot=rot, k_rot=rot)
     cos_rot = float(torch.nn.functional.cosine_similarity(out8r.float().flatten(), out16.float().flatten(), dim=0))
+    # rotation + power-of-two scales: with the outliers spread, the faster recipe loses no accuracy
+    rotp_ms, _ = time_steps(lambda: f8.fp8_attention_forward(q, k, v, q_rot=rot, k_rot=rot, recipe="pow2"), steps, warmup)
+    out8r = f8.fp8_attention_forward(q, k, v, q_rot=rot, k_rot=rot, recipe="pow2")
+    cos_rotp = float(torch.nn.functional.cosine_similarity(out8r.float().flatten(), out16.float().flatten(), dim=0))
     f = attn_flops(cfg)
     bm, km, qm, em = median(bf16_ms), median(kern_ms), median(quant_ms), median(e2e_ms)
     # quantisation pass: read q, k once and v twice (maximum, then quantise), write one byte per element
     quant_bytes = (4 * 2 + 3 * 1) * cfg["N"] * cfg["S"] * cfg["D"]
-    return {"workload": "FP8 attention B1 N40 S32760 D128, N(0,1) with 1% x8 outliers; Q,K per-128-token scales, "
-                        "V per-channel, P e4m3 per tile",
+    return {"workload": "FP8 attention B1 N40 S32760 D128, N(0,1) with 1% x8 outliers; Q,K per-128-token scales "
+                        "(amax/448), V per-channel, P e4m3 per tile",
             "bf16_ms": bm, "bf16_tflops": f / bm / 1e9,
             "fp8_kernel_ms": km, "fp8_kernel_tflops": f / km / 1e9, "fp8_kernel_frac_of_fp8_peak": f / km / 1e9 / PEAK_FP8_TFLOPS,
             "fp8_kernel_speedup_vs_bf16": bm / km,
             "quant_pass_ms": qm, "quant_pass_gbs": quant_bytes / qm / 1e6,
             "fp8_end_to_end_ms": em, "fp8_end_to_end_speedup_vs_bf16": bm / em,
             "cosine_fp8_vs_unquantised_bf16_kernel": cos,
+            "pow2_recipe_kernel_ms": median(pkern_ms), "pow2_recipe_kernel_speedup_vs_bf16": bm / median(pkern_ms),
+            "pow2_recipe_end_to_end_ms": median(pe2e_ms), "pow2_recipe_end_to_end_speedup_vs_bf16": bm / median(pe2e_ms),
+            "pow2_recipe_cosine_vs_unquantised_bf16_kernel": cos_p,
             "rotated_end_to_end_ms": median(rot_ms), "rotated_end_to_end_speedup_vs_bf16": bm / median(rot_ms),
             "rotate_quant_qk_fused_ms": median(rq_ms), "rotate_quant_qk_matmul_then_quant_ms": median(mm_ms),
-            "cosine_rotated_fp8_vs_unquantised_bf16_kernel": cos_rot}
+            "cosine_rotated_fp8_vs_unquantised_bf16_kernel": cos_rot,
+            "rotated_pow2_end_to_end_ms": median(rotp_ms), "rotated_pow2_end_to_end_speedup_vs_bf16": bm / median(rotp_ms),
+            "cosine_rotated_pow2_fp8_vs_unquantised_bf16_kernel": cos_rotp}
 
 
 def extra_gemm(device, steps, warmup):

@@ -41,6 +41,17 @@ __device__ __forceinline__ int pack4_e4m3_noclamp(float a, float b, float c, flo
   return w;
 }
 
+// Quantisation scale of a block with maximum magnitude amax: amax / 448, or (pow2) the smallest power of two
+// that is not below it, so that the scale can later be applied by the matrix instruction's exponent operand.
+__device__ __forceinline__ float block_scale(float amax, int pow2) {
+  if (!(amax > 0.f)) return 1.0f;
+  const float sc = __fdiv_rn(amax, kE4M3Max);
+  if (!pow2) return sc;
+  const unsigned bits = __builtin_bit_cast(unsigned, sc);
+  const unsigned e = max((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u), 1u);  // at least 2^-126
+  return __builtin_bit_cast(float, e << 23);
+}
+
 template <int DT>
 __device__ __forceinline__ void load8(const typename Elem<DT>::type* p, float (&f)[8]) {
   union { i32x4_t v; typename Elem<DT>::type e[8]; } u;
@@ -64,7 +75,7 @@ __device__ __forceinline__ float block_max_256(float v, float* red) {
 template <int DT>
 __global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsigned char* q, float* scale,
                                                           long long sb, long long sn, long long ss, int N, int S,
-                                                          int bs) {
+                                                          int bs, float prescale, int pow2) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using T = typename Elem<DT>::type;
   __shared__ float red[4];
@@ -79,17 +90,17 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsign
     float f[8];
     load8<DT>(x + (long long)(row0 + r) * ss + c16 * 8, f);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(__fmul_rn(f[j], prescale)));
   }
   amax = block_max_256(amax, red);
-  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  const float sc = block_scale(amax, pow2);
   if (threadIdx.x == 0) scale[(long long)bn * nblk + blk] = sc;
   unsigned char* qo = q + ((long long)bn * S + row0) * 128 + c16 * 8;
   for (int r = rgrp; r < rows; r += 16) {
     float f[8];
     load8<DT>(x + (long long)(row0 + r) * ss + c16 * 8, f);   // second read hits L2
 #pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn(f[j], sc);
+    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn(__fmul_rn(f[j], prescale), sc);
     i32x2_t w = {pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
     *(i32x2_t*)(qo + (long long)r * 128) = w;
   }
@@ -100,7 +111,8 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const void* x_, unsign
 // at once (more requests in flight than the row loop above) and quantises them without a second read.
 template <int DT>
 __global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, unsigned char* q, float* scale,
-                                                             long long sb, long long sn, long long ss, int N, int S) {
+                                                             long long sb, long long sn, long long ss, int N, int S,
+                                                             float prescale, int pow2) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using T = typename Elem<DT>::type;
   __shared__ float red[4];
@@ -121,9 +133,9 @@ __global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, uns
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf((float)u[i].e[j]));
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(__fmul_rn((float)u[i].e[j], prescale)));
   amax = block_max_256(amax, red);
-  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  const float sc = block_scale(amax, pow2);
   if (threadIdx.x == 0) scale[(long long)bn * nblk + blk] = sc;
   unsigned char* qo = q + ((long long)bn * S + row0) * 128 + c16 * 8;
 #pragma unroll
@@ -131,7 +143,7 @@ __global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, uns
     const int r = rgrp + 16 * i;
     float f[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn((float)u[i].e[j], sc);
+    for (int j = 0; j < 8; ++j) f[j] = __fdiv_rn(__fmul_rn((float)u[i].e[j], prescale), sc);
     const i32x2_t w = {pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
     if (r < rows) *(i32x2_t*)(qo + (long long)r * 128) = w;
   }
@@ -149,7 +161,7 @@ __global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, uns
 template <int DT>
 __global__ __launch_bounds__(256) void rot_block_quant_kernel(const void* x_, const void* rot_t_, unsigned char* q,
                                                               float* scale, long long sb, long long sn, long long ss,
-                                                              int N, int S) {
+                                                              int N, int S, float prescale, int pow2) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
   using T = typename E::type;
@@ -198,11 +210,11 @@ __global__ __launch_bounds__(256) void rot_block_quant_kernel(const void* x_, co
   for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      acc[nb][r] = (float)E::from_float(acc[nb][r]);
+      acc[nb][r] = __fmul_rn((float)E::from_float(acc[nb][r]), prescale);
       amax = fmaxf(amax, fabsf(acc[nb][r]));
     }
   amax = block_max_256(amax, red);
-  const float sc = amax > 0.f ? __fdiv_rn(amax, kE4M3Max) : 1.0f;
+  const float sc = block_scale(amax, pow2);
   if (tid == 0) scale[(long long)bn * nblk + blk] = sc;
   if (ok) {
     unsigned char* qo = q + ((long long)bn * S + tok) * 128;
@@ -337,7 +349,11 @@ constexpr float kPShift = 4.0f;
 
 // 8 waves x 32 query rows, 128-key tiles, K tile [key][128 B] and V^T tile [channel][128 B] in LDS
 // (16 KiB each, double buffered); 16-byte chunk c of row r is stored at chunk c ^ ((r >> 1) & 7).
-template <int DT>
+// P2 (log2 domain): q_scale and k_scale are powers of two and the query codes already carry the softmax scale
+// times log2(e).  The two scales then go into the exponent operands of the scaled matrix instruction and the
+// score accumulators are seeded with kPShift - m, so the matrix core delivers s - m + kPShift and the softmax is
+// exp2 and rounding alone (no multiply-add per score).
+template <int DT, bool P2>
 __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
@@ -376,7 +392,9 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   }
   // all 32 rows of a wave lie in one 128-row scale block
   const int qblk = min((q0 + wave * 32) >> 7, qblocks - 1);
-  const float q_sc = p.q_scale[(long long)bn * qblocks + qblk] * p.scale_log2;
+  const float q_sc_raw = p.q_scale[(long long)bn * qblocks + qblk];
+  const float q_sc = q_sc_raw * p.scale_log2;
+  const int q_exp = (int)((__builtin_bit_cast(unsigned, q_sc_raw) >> 23) & 0xffu);  // E8M0 code of a power of two
   const float* k_sc = p.k_scale + (long long)bn * kblocks;
 
   f32x16_t oacc[4];
@@ -384,7 +402,11 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-  float m_run = -INFINITY;
+  float m_run = P2 ? 0.f : -INFINITY;
+  f32x16_t negm;  // P2: kPShift - m_run in every slot, the seed of the score accumulators
+#pragma unroll
+  for (int r = 0; r < 16; ++r) negm[r] = kPShift;
+  bool first = true;
 
   // ---- LDS-DMA staging: one instruction = 8 rows x 128 bytes ----------------------------------------------------
   const unsigned char* kg = p.k8 + (long long)bn * p.Skv * 128;
@@ -442,10 +464,13 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 
     // ---- S^T = K Q^T (fp8, unscaled form of the scaled MFMA) ---------------------------------------------------
     f32x16_t sacc[4];
+    const int k_exp = (int)((__builtin_bit_cast(unsigned, k_sc_cur) >> 23) & 0xffu);
+    if (!P2) {
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+      for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+        for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+    }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -454,7 +479,11 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
         const i32x4_t lo = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h) ^ swz) << 4));
         const i32x4_t hi = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h + 1) ^ swz) << 4));
         const i32x8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
+        if (P2)
+          sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], ks == 0 ? negm : sacc[kb], 0, 0, 0,
+                                                                     k_exp, 0, q_exp);
+        else
+          sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
       }
     }
 
@@ -475,6 +504,38 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+    i32x8_t pf[2];
+    if (P2) {
+      // sacc = s - m_run + kPShift; the reference maximum moves when a row exceeds it by more than kTau8
+      mx = half_max(mx) - kPShift;
+      if (first || __builtin_amdgcn_ballot_w64(mx > kTau8) != 0) {
+        float delta = first ? mx : fmaxf(mx, 0.f);
+        delta = (delta == -INFINITY) ? 0.f : delta;
+        const float alpha = fast_exp2(-delta);
+        m_run += delta;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) negm[r] = kPShift - m_run;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[kb][r] -= delta;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lacc[r] *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+      }
+      first = false;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+          pf[kb >> 1][(kb & 1) * 4 + g4] =
+              pack4_e4m3_noclamp(fast_exp2(sacc[kb][4 * g4]), fast_exp2(sacc[kb][4 * g4 + 1]),
+                                 fast_exp2(sacc[kb][4 * g4 + 2]), fast_exp2(sacc[kb][4 * g4 + 3]));
+      }
+    } else {
     mx = half_max(mx) * c;
     if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau8) != 0) {
       const float m_new = fmaxf(m_run, mx);
@@ -488,7 +549,6 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
         for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
     }
     const float mc = (m_run == -INFINITY ? 0.f : m_run) - kPShift;
-    i32x8_t pf[2];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
@@ -498,6 +558,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
             fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 2], c, -mc)),
             fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 3], c, -mc)));
     }
+    }  // !P2
 
     // ---- O^T += V^T P^T (fp8), row sums ---------------------------------------------------------------------------
 #pragma unroll
@@ -559,8 +620,9 @@ using namespace msd;
 extern "C" {
 
 int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int B, int N, int S, int D,
-                            long long x_sb, long long x_sn, long long x_ss, int block_size, hipStream_t stream) {
-  if (!x || !q || !scale || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+                            long long x_sb, long long x_sn, long long x_ss, int block_size, float prescale,
+                            int pow2_scale, hipStream_t stream) {
+  if (!x || !q || !scale || B <= 0 || N <= 0 || S <= 0 || !(prescale > 0.f)) return MSD_ERR_BAD_ARG;
   if (D != 128) return MSD_ERR_UNSUPPORTED;
   if (block_size != 128 && block_size != 256 && block_size != 512) return MSD_ERR_BAD_ARG;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
@@ -569,26 +631,27 @@ int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int
   if (block_size == 128) {
     if (dtype == MSD_DTYPE_BF16)
       hipLaunchKernelGGL(block_quant128_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale,
-                         x_sb, x_sn, x_ss, N, S);
+                         x_sb, x_sn, x_ss, N, S, prescale, pow2_scale ? 1 : 0);
     else
       hipLaunchKernelGGL(block_quant128_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale,
-                         x_sb, x_sn, x_ss, N, S);
+                         x_sb, x_sn, x_ss, N, S, prescale, pow2_scale ? 1 : 0);
     return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
   }
   if (dtype == MSD_DTYPE_BF16)
     hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
-                       x_sn, x_ss, N, S, block_size);
+                       x_sn, x_ss, N, S, block_size, prescale, pow2_scale ? 1 : 0);
   else
     hipLaunchKernelGGL(block_quant_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, (unsigned char*)q, scale, x_sb,
-                       x_sn, x_ss, N, S, block_size);
+                       x_sn, x_ss, N, S, block_size, prescale, pow2_scale ? 1 : 0);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
 // y = x @ rot (rot_t = rot transposed, [128][128] contiguous, same 16-bit type as x), rounded to the
 // 16-bit type, then quantised per (head, 128 tokens): codes [B][N][S][128], scale [B][N][ceil(S/128)].
 int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float* scale, int dtype, int B, int N, int S,
-                                int D, long long x_sb, long long x_sn, long long x_ss, hipStream_t stream) {
-  if (!x || !rot_t || !q || !scale || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+                                int D, long long x_sb, long long x_sn, long long x_ss, float prescale, int pow2_scale,
+                                hipStream_t stream) {
+  if (!x || !rot_t || !q || !scale || B <= 0 || N <= 0 || S <= 0 || !(prescale > 0.f)) return MSD_ERR_BAD_ARG;
   if (D != 128) return MSD_ERR_UNSUPPORTED;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
   if ((((uintptr_t)x | (uintptr_t)rot_t) & 15) || ((uintptr_t)q & 3) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
@@ -596,10 +659,10 @@ int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float
   if (grid.y > 65535) return MSD_ERR_UNSUPPORTED;
   if (dtype == MSD_DTYPE_BF16)
     hipLaunchKernelGGL(rot_block_quant_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, x, rot_t, (unsigned char*)q,
-                       scale, x_sb, x_sn, x_ss, N, S);
+                       scale, x_sb, x_sn, x_ss, N, S, prescale, pow2_scale ? 1 : 0);
   else
     hipLaunchKernelGGL(rot_block_quant_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, x, rot_t, (unsigned char*)q,
-                       scale, x_sb, x_sn, x_ss, N, S);
+                       scale, x_sb, x_sn, x_ss, N, S, prescale, pow2_scale ? 1 : 0);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
@@ -636,7 +699,7 @@ int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, in
 int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
                                const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
                                int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,
-                               hipStream_t stream) {
+                               int log2_domain, hipStream_t stream) {
   if (!q8 || !k8 || !v8t || !q_scale || !k_scale || !v_scale || !out) return MSD_ERR_BAD_ARG;
   if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return MSD_ERR_BAD_ARG;
   if (D != 128 || !(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
@@ -655,13 +718,27 @@ int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, 
   const int q_tiles = (Sq + 255) / 256;
   const int total = B * N * q_tiles;
   const int grid = (total + 7) / 8 * 8;
+  if (log2_domain) {
+    if (out_dtype == MSD_DTYPE_BF16) {
+      auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16, true>;
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+        return MSD_ERR_LAUNCH;
+      hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
+    } else {
+      auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16, true>;
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+        return MSD_ERR_LAUNCH;
+      hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
+    }
+    return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+  }
   if (out_dtype == MSD_DTYPE_BF16) {
-    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16>;
+    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16, false>;
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
       return MSD_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
   } else {
-    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16>;
+    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16, false>;
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
       return MSD_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);

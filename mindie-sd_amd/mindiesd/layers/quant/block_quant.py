@@ -6,9 +6,10 @@ from ...utils.exception import ParametersInvalid
 from ..flash_attn.hip_flash_attn import HEAD_DIM, _strides_bns
 
 
-def _block_quant(x, block_size, layout):
+def _block_quant(x, block_size, layout, prescale=1.0, pow2=False):
     """x 4-D bf16/fp16 GPU tensor in ``layout`` -> (uint8 E4M3 codes [B,N,S,D] contiguous, fp32 scale
-    [B,N,ceil(S/block_size)])."""
+    [B,N,ceil(S/block_size)]).  ``prescale`` multiplies x first; ``pow2`` rounds each scale up to a power of two
+    (x * prescale ~ codes * scale either way)."""
     if x.dtype not in _native.DTYPE_CODE or not x.is_cuda:
         raise ParametersInvalid(f"fa block quant needs a bf16/fp16 GPU tensor, but got {x.dtype} on {x.device}.")
     if x.shape[-1] != HEAD_DIM:
@@ -23,13 +24,13 @@ def _block_quant(x, block_size, layout):
     with torch.cuda.device(x.device):
         rc = _native.lib().mindiesd_fa_block_quant(x.data_ptr(), q.data_ptr(), scale.data_ptr(),
                                                    _native.DTYPE_CODE[x.dtype], b, n, s, HEAD_DIM,
-                                                   *_strides_bns(x, layout), block_size,
-                                                   _native.stream_ptr(x.device))
+                                                   *_strides_bns(x, layout), block_size, float(prescale),
+                                                   int(bool(pow2)), _native.stream_ptr(x.device))
     _native.check(rc, "mindiesd_fa_block_quant")
     return q, scale
 
 
-def _rot_block_quant(x, rot, layout):
+def _rot_block_quant(x, rot, layout, prescale=1.0, pow2=False):
     """(x @ rot) rounded to x.dtype, then quantised per (head, 128 tokens) in one pass over x.
     x 4-D bf16/fp16 GPU tensor in ``layout``, rot [128, 128]; returns (uint8 codes [B,N,S,D], fp32 scale
     [B,N,ceil(S/128)])."""
@@ -47,7 +48,8 @@ def _rot_block_quant(x, rot, layout):
     with torch.cuda.device(x.device):
         rc = _native.lib().mindiesd_fa_rot_block_quant(x.data_ptr(), rot_t.data_ptr(), q.data_ptr(), scale.data_ptr(),
                                                        _native.DTYPE_CODE[x.dtype], b, n, s, HEAD_DIM,
-                                                       *_strides_bns(x, layout), _native.stream_ptr(x.device))
+                                                       *_strides_bns(x, layout), float(prescale), int(bool(pow2)),
+                                                       _native.stream_ptr(x.device))
     _native.check(rc, "mindiesd_fa_rot_block_quant")
     return q, scale
 

@@ -33,9 +33,15 @@ def quantize_v_per_channel(value, layout="BNSD"):
     return v8t, vscale
 
 
-def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_dtype=torch.bfloat16, layout="BNSD"):
+LOG2E = 1.4426950408889634
+
+
+def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_dtype=torch.bfloat16, layout="BNSD",
+                            log2_domain=False):
     """Attention on already quantised operands (see ``quantize_v_per_channel`` and ``_block_quant``
-    with block 128).  Output [B,N,S,128] ('BNSD') or [B,S,N,128] ('BSND') in ``out_dtype``."""
+    with block 128).  Output [B,N,S,128] ('BNSD') or [B,S,N,128] ('BSND') in ``out_dtype``.
+    ``log2_domain``: the query was quantised with ``prescale = scale * log2(e)`` and both q and k with
+    power-of-two scales; ``scale`` is then not used."""
     b, n, sq, d = q8.shape
     skv = k8.shape[2]
     shape = (b, n, sq, d) if layout == "BNSD" else (b, sq, n, d)
@@ -44,15 +50,22 @@ def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_d
         rc = _native.lib().mindiesd_fp8_attention_fwd(
             q8.data_ptr(), k8.data_ptr(), v8t.data_ptr(), q_scale.data_ptr(), k_scale.data_ptr(), v_scale.data_ptr(),
             out.data_ptr(), _native.DTYPE_CODE[out_dtype], b, n, sq, skv, d, *_strides_bns(out, layout),
-            float(scale), _native.stream_ptr(q8.device))
+            float(scale), int(bool(log2_domain)), _native.stream_ptr(q8.device))
     _native.check(rc, "mindiesd_fp8_attention_fwd")
     return out
 
 
-def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None):
+def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None, recipe="amax"):
     """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``.
     ``q_rot`` / ``k_rot`` ([128, 128]): query @ q_rot and key @ k_rot are formed inside the quantisation
-    pass (the rotated tensors are never written)."""
+    pass (the rotated tensors are never written).
+    ``recipe``: 'amax' (default, the reference's dynamic block quantisation) - Q and K block scales amax/448, the
+    scores are rescaled in the softmax; 'pow2' - block scales rounded up to powers of two and the softmax scale
+    folded into the query before quantisation, so the matrix instruction applies the scales through its exponent
+    operands and the softmax needs no multiply (about 4 % faster).  On inputs without outliers both give the same
+    accuracy; with amax/448 the largest element of every block is encoded exactly (code 448), which 'pow2' gives
+    up, and on inputs whose softmax is decided by a few outliers that costs accuracy (cosine 0.979 against 0.987
+    at 32760 tokens with 1 % of the elements scaled by 8)."""
     for name, t in (("query", query), ("key", key), ("value", value)):
         if not isinstance(t, torch.Tensor) or t.dim() != 4:
             raise ParametersInvalid(f"The input {name} must be a 4-D torch.Tensor.")
@@ -66,7 +79,13 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=No
         raise ParametersInvalid("fp8 attention needs the same batch and head count for query and key/value.")
     if scale is None:
         scale = query.shape[-1] ** -0.5
-    q8, qs = _block_quant(query, 128, layout) if q_rot is None else _rot_block_quant(query, q_rot, layout)
-    k8, ks = _block_quant(key, 128, layout) if k_rot is None else _rot_block_quant(key, k_rot, layout)
+    if recipe not in ("pow2", "amax"):
+        raise ParametersInvalid(f"recipe must be 'pow2' or 'amax', but got {recipe}.")
+    p2 = recipe == "pow2"
+    pre = float(scale) * LOG2E if p2 else 1.0
+    q8, qs = (_block_quant(query, 128, layout, pre, p2) if q_rot is None
+              else _rot_block_quant(query, q_rot, layout, pre, p2))
+    k8, ks = (_block_quant(key, 128, layout, 1.0, p2) if k_rot is None
+              else _rot_block_quant(key, k_rot, layout, 1.0, p2))
     v8t, vs = quantize_v_per_channel(value, layout)
-    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout)
+    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout, log2_domain=p2)

@@ -60,10 +60,19 @@ def e4m3_round(x):
 
 
 # ---- block quantisation of attention operands ----------------------------------------------------------
-def dynamic_block_quant(x, row_block=128, col_block=128):
+def pow2_ceil(sc):
+    """Smallest power of two >= sc (fp32 array of positive normal numbers; at least 2^-126)."""
+    m, e = np.frexp(sc.astype(np.float32))          # sc = m * 2^e, m in [0.5, 1)
+    e = np.where(m == 0.5, e - 1, e)
+    return np.ldexp(np.float32(1.0), np.maximum(e, -126)).astype(np.float32)
+
+
+def dynamic_block_quant(x, row_block=128, col_block=128, prescale=1.0, pow2=False):
     """[..., S, D] -> (codes uint8 same shape, scale fp32 [..., ceil(S/row_block), ceil(D/col_block)]).
-    One scale per (row_block tokens x col_block channels) tile: scale = amax/448, q = e4m3(x/scale)."""
-    xf = x.float().numpy()
+    One scale per (row_block tokens x col_block channels) tile: scale = amax/448, q = e4m3(x/scale).
+    ``prescale`` multiplies x first (one fp32 rounding); ``pow2`` rounds the scale up to a power of two - the
+    recipe of the log2-domain FP8 attention kernel (not in the reference)."""
+    xf = (x.float().numpy() * np.float32(prescale)).astype(np.float32)
     s, d = xf.shape[-2:]
     nb_r, nb_c = math.ceil(s / row_block), math.ceil(d / col_block)
     codes = np.zeros(xf.shape, dtype=np.uint8)
@@ -74,17 +83,19 @@ def dynamic_block_quant(x, row_block=128, col_block=128):
             blk = xf[..., rs, cs]
             amax = np.abs(blk).max(axis=(-1, -2)).astype(np.float32)
             sc = np.where(amax > 0, amax / np.float32(E4M3_MAX), np.float32(1.0)).astype(np.float32)
+            if pow2:
+                sc = np.where(amax > 0, pow2_ceil(sc), np.float32(1.0)).astype(np.float32)
             scale[..., i, j] = sc
             codes[..., rs, cs] = e4m3_encode(blk / sc[..., None, None])
     return torch.from_numpy(codes), torch.from_numpy(scale)
 
 
-def rot_block_quant(x, rot, row_block=128):
+def rot_block_quant(x, rot, row_block=128, prescale=1.0, pow2=False):
     """FP8RotateQuantFA's first two steps (mindiesd/quantization/layer.py:284-296) on the CPU:
     ``torch.matmul(x, rot)`` in the 16-bit input type (fp32 accumulation, one rounding), then
     ``dynamic_block_quant`` over (row_block tokens x all channels)."""
     y = torch.matmul(x.float(), rot.to(x.dtype).float()).to(x.dtype)
-    return dynamic_block_quant(y, row_block, x.shape[-1])
+    return dynamic_block_quant(y, row_block, x.shape[-1], prescale, pow2)
 
 
 def dequant_block(codes, scale, row_block=128, col_block=128):
@@ -102,7 +113,7 @@ def per_channel_quant(v):
     return torch.from_numpy(e4m3_encode(vf / sc[..., None, :])), torch.from_numpy(sc)
 
 
-def fp8_attention(query, key, value, scale=None):
+def fp8_attention(query, key, value, scale=None, pow2=False):
     """FP8 attention of the Wan2.1-14B 480p workload, BNSD: Q and K quantised per (head, 128-token
     block) over all channels, V per (head, channel); everything is dequantised and run through plain
     softmax(scale QK^T)V in fp32; bf16-typed output.  (The quantise -> dequantise path: the GPU kernel
@@ -111,8 +122,15 @@ def fp8_attention(query, key, value, scale=None):
     d = query.shape[-1]
     if scale is None:
         scale = d ** -0.5
-    qc, qs = dynamic_block_quant(query, 128, d)
-    kc, ks = dynamic_block_quant(key, 128, d)
+    if pow2:
+        # log2-domain recipe: the query carries scale * log2(e), block scales are powers of two; the dequantised
+        # scores are then in log2 units, i.e. ln(2) stands where the softmax scale stood
+        qc, qs = dynamic_block_quant(query, 128, d, scale * 1.4426950408889634, True)
+        kc, ks = dynamic_block_quant(key, 128, d, 1.0, True)
+        scale = math.log(2.0)
+    else:
+        qc, qs = dynamic_block_quant(query, 128, d)
+        kc, ks = dynamic_block_quant(key, 128, d)
     vc, vs = per_channel_quant(value)
     qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, 128, d)
     vd = torch.from_numpy(e4m3_decode(vc.numpy())) * vs[..., None, :]

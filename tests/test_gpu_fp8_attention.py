@@ -72,13 +72,35 @@ def test_v_per_channel_quant_bit_exact(cuda):
     assert (got[:, :, 333:] & 0x7f == 0).all(), "padding keys must be zero"
 
 
+@pytest.mark.parametrize("layout", ["BNSD", "BSND"])
+@pytest.mark.parametrize("prescale", [1.0, 0.12751743])
+def test_pow2_block_quant_bit_exact(cuda, prescale, layout):
+    """Power-of-two block scales (+ a factor folded into x): the recipe of the log2-domain attention kernel."""
+    from mindiesd.layers.quant.block_quant import _block_quant
+    x = _outlier_inputs((1, 3, 1000, 128), seed=17)[0]
+    x[0, 1, 256:384] = 0
+    x[0, 2, :128] = 448.0 * 4                 # amax / 448 already a power of two: must not be doubled
+    xin = x if layout == "BNSD" else x.transpose(1, 2).contiguous()
+    q, scale = _block_quant(xin.to(cuda), 128, layout, prescale, True)
+    codes, want_scale = oq.dynamic_block_quant(x, 128, 128, prescale, True)
+    assert torch.equal(scale.cpu(), want_scale[..., 0])
+    frac = np.frexp(scale.cpu().numpy())[0]
+    assert (frac == 0.5).all(), "scales must be powers of two"
+    got = q.cpu()
+    zero = ((got & 0x7f) == 0) & ((codes & 0x7f) == 0)
+    assert bool(((got == codes) | zero).all())
+    if prescale == 1.0:
+        assert scale[0, 2, 0].item() == 4.0
+
+
+@pytest.mark.parametrize("recipe", ["pow2", "amax"])
 @pytest.mark.parametrize("layout,s", [("BNSD", 1024), ("BNSD", 1100), ("BSND", 700)])
-def test_fp8_attention_vs_oracle(cuda, layout, s):
+def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
     from mindiesd.layers.quant import fp8_attention_forward
     q, k, v = _outlier_inputs((1, 3, s, 128), seed=s)
-    want = oq.fp8_attention(q, k, v)
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2")
     args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
-    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout).cpu()
+    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout, recipe=recipe).cpu()
     out = out if layout == "BNSD" else out.transpose(1, 2)
     assert out.dtype == torch.bfloat16 and out.shape == q.shape
     cos = cosine(out, want)

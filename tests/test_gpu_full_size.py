@@ -94,11 +94,14 @@ def test_fp8_attention_wan14b_480p(cuda):
     assert bool(((deq - k.float()).abs() <= step * 1.0001).all())
     del kp, deq, step, codes
     # two query blocks of two heads against the quantise -> dequantise oracle (cosine >= 0.999)
+    # (each recipe against the oracle of the same recipe)
+    out_p2 = fp8_attention_forward(q, k, v, layout="BNSD", recipe="pow2")
     for head in (0, 39):
         qs = q[:, head:head + 1, 128 * 100: 128 * 102].cpu()
-        want = oq.fp8_attention(qs, k[:, head:head + 1].cpu(), v[:, head:head + 1].cpu())
-        got = out[:, head:head + 1, 128 * 100: 128 * 102].cpu()
-        assert oa.cosine(got, want) >= 0.999, oa.cosine(got, want)
+        for res, p2 in ((out, False), (out_p2, True)):
+            want = oq.fp8_attention(qs, k[:, head:head + 1].cpu(), v[:, head:head + 1].cpu(), pow2=p2)
+            got = res[:, head:head + 1, 128 * 100: 128 * 102].cpu()
+            assert oa.cosine(got, want) >= 0.999, (p2, oa.cosine(got, want))
 
 
 def test_mxfp8_gemm_swiglu_ffn_shape(cuda):

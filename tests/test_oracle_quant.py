@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from oracle import quant as oq
+from oracle.attention import attention_math, cosine
 
 
 def test_e4m3_all_codes_round_trip_and_match_torch():
@@ -102,3 +103,44 @@ def test_fp8_attention_close_to_unquantised():
     assert out.dtype == torch.bfloat16
     for n in range(2):
         assert cosine(out[0, n], attention_fp64(q[0, n], k[0, n], v[0, n], 128 ** -0.5)) > 0.995
+
+
+# ---- power-of-two block scales (recipe of the log2-domain FP8 attention kernel; not in the reference) -------------
+def test_pow2_ceil_closed_forms():
+    sc = np.array([1.0, 1.0000001, 0.75, 0.5, 0.50000006, 3.0, 4.0, 2.0 ** -20, 1e-45], dtype=np.float32)
+    want = np.array([1.0, 2.0, 1.0, 0.5, 1.0, 4.0, 4.0, 2.0 ** -20, 2.0 ** -126], dtype=np.float32)
+    assert np.array_equal(oq.pow2_ceil(sc), want)
+
+
+def test_pow2_block_quant_properties():
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(2, 300, 128, generator=g) * 3).to(torch.bfloat16)
+    x[0, :128] = 0
+    codes, scale = oq.dynamic_block_quant(x, 128, 128, pow2=True)
+    _, plain = oq.dynamic_block_quant(x, 128, 128)
+    s, p = scale.numpy(), plain.numpy()
+    nz = p != 1.0
+    assert (np.frexp(s)[0] == 0.5).all()                       # powers of two
+    assert (s[nz] >= p[nz]).all() and (s[nz] < 2 * p[nz]).all()  # smallest one not below amax / 448
+    assert s[0, 0, 0] == 1.0 and (codes[0, :128].numpy() & 0x7f == 0).all()
+    deq = oq.dequant_block(codes, scale, 128, 128)
+    rel = (deq - x.float()).abs() / x.float().abs().clamp_min(1e-3)
+    big = x.float().abs() > 0.05 * x.float().abs().amax(dim=(-1, -2), keepdim=True)
+    assert rel[big].max() <= 2.0 ** -4 + 1e-6                  # E4M3: 3 mantissa bits, half an ulp
+    assert int(codes.max()) <= 0x7e | 0x80 and (codes.numpy() & 0x7f).max() <= 0x7e  # never NaN / beyond 448
+
+
+def test_prescale_by_a_power_of_two_only_moves_the_scale():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(1, 256, 128, generator=g).to(torch.bfloat16)
+    c1, s1 = oq.dynamic_block_quant(x, 128, 128, 1.0, True)
+    c2, s2 = oq.dynamic_block_quant(x, 128, 128, 0.125, True)
+    assert torch.equal(c1, c2) and torch.equal(s2, s1 * 0.125)
+
+
+def test_fp8_attention_recipes_agree_with_each_other_and_with_plain_attention():
+    g = torch.Generator().manual_seed(7)
+    q, k, v = (torch.randn(1, 2, 384, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    a, b = oq.fp8_attention(q, k, v), oq.fp8_attention(q, k, v, pow2=True)
+    ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=True)
+    assert cosine(a, b) > 0.997 and cosine(b, ref) > 0.995 and cosine(a, ref) > 0.995
