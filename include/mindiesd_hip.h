@@ -76,7 +76,8 @@ void mindiesd_set_dense_variant(int variant);
 /* ---- block-sparse attention ------------------------------------------------------------------------
  * Query block i (128 rows) of (b, n) attends to the 128-key blocks blk_idx[b][n][i][0 .. blk_cnt[b][n][i])
  * (ascending ids, int32, row pitch kb_stride); an empty list gives zeros.  `order` (optional,
- * [B*N*ceil(Sq/128)]) is the sequence in which query blocks are dispatched.
+ * [B*N*ceil(Sq/128)], a permutation of the query block numbers (b*N + n)*ceil(Sq/128) + i) is the sequence
+ * in which query blocks are dispatched: workgroup j takes block order[j].
  * Replaces aclnnBlockSparseAttention / aclnnRainFusionAttention behind
  * torch.ops.mindiesd.block_sparse_attention / rainfusionattention
  * (csrc/plugin/block_sparse_attention.cpp:31-121, csrc/plugin/rainfusionattention.cpp:27-64). */

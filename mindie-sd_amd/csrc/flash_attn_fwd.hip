@@ -132,9 +132,11 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int total = p.B * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
   int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
-  if (work >= total) return;
-  if (SPARSE && p.order) work = p.order[blockIdx.x < total ? blockIdx.x : 0];
-  if (SPARSE && p.order && blockIdx.x >= total) return;
+  if (SPARSE && p.order) {  // caller's work order: workgroup i takes entry i of the table
+    if ((int)blockIdx.x >= total) return;
+    work = p.order[blockIdx.x];
+  }
+  if (work < 0 || work >= total) return;
   const int bn = work / q_tiles;
   int qt = work - bn * q_tiles;
   if (MODE && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first

@@ -166,6 +166,31 @@ def test_block_sparse_attention_op_vs_oracle(cuda, s, dtype):
     assert (out[:, :, 128:256] == 0).all(), "query block with no selected key block must be zero"
 
 
+def test_block_sparse_dispatch_order_table(cuda):
+    """The optional work-order table of the C entry point only changes which workgroup takes which query block:
+    any permutation gives the bits of the default order (27 query blocks, not a multiple of the 8 XCDs)."""
+    from mindiesd import _native
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    from mindiesd.layers.flash_attn.hip_flash_attn import _strides_bns
+    s, n = 1100, 3
+    q, k, v = (_rand((1, n, s, 128), seed=i).to(cuda) for i in (14, 15, 16))
+    nb = (s + 127) // 128
+    idx, cnt = rf.mask_to_lists(_random_block_mask(1, n, nb, nb, 0.5, seed=7).to(cuda))
+    want = rf.block_sparse_attention_lists(q, k, v, idx, cnt, 128 ** -0.5, "BNSD")
+    g = torch.Generator().manual_seed(3)
+    for order in (torch.randperm(n * nb, generator=g), torch.arange(n * nb - 1, -1, -1)):
+        order = order.to(torch.int32).to(cuda)
+        out = torch.full_like(q, float("nan"))
+        with torch.cuda.device(cuda):
+            rc = _native.lib().mindiesd_block_sparse_attention_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None, _native.DTYPE_CODE[q.dtype], 1, n, n, s, s,
+                128, *_strides_bns(q, "BNSD"), *_strides_bns(k, "BNSD"), *_strides_bns(v, "BNSD"),
+                *_strides_bns(out, "BNSD"), 128 ** -0.5, idx.data_ptr(), cnt.data_ptr(), idx.shape[3], order.data_ptr(),
+                _native.stream_ptr(cuda))
+        assert rc == 0
+        assert torch.equal(out, want)
+
+
 def test_full_mask_equals_dense(cuda):
     """sparsity 0 == dense attention (tests/layers/flash_attn/test_sparse_attention.py:73-122)."""
     import mindiesd
