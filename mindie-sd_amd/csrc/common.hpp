@@ -41,6 +41,9 @@ struct Elem<MSD_DTYPE_BF16> {
   static __device__ __forceinline__ f32x16_t mfma32(x8 a, x8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x4_t mfma16(x8 a, x8 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ type from_float(float f) { return (__bf16)f; }
   // acc + sum of the 8 elements (v_dot2_f32_bf16 against ones)
   static __device__ __forceinline__ float sum8(x8 v, float acc) {
@@ -60,6 +63,9 @@ struct Elem<MSD_DTYPE_F16> {
   typedef f16x4_t x4;
   static __device__ __forceinline__ f32x16_t mfma32(x8 a, x8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4_t mfma16(x8 a, x8 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ type from_float(float f) { return (_Float16)f; }
   static __device__ __forceinline__ float sum8(x8 v, float acc) {
@@ -125,6 +131,27 @@ __device__ __forceinline__ float half_sum(float v) {
   float lo, hi;
   half_swap(v, lo, hi);
   return lo + hi;
+}
+
+// The same across the four 16-lane rows of a wavefront: v_permlane16_swap exchanges the odd rows of its first
+// operand with the even rows of its second, so with both holding v one result has rows (0, 0, 2, 2) of v and
+// the other rows (1, 1, 3, 3); combining them and then the two halves leaves the result of all four rows in
+// every lane.
+__device__ __forceinline__ void row_swap(float v, float& even, float& odd) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  even = a;
+  odd = b;
+}
+__device__ __forceinline__ float quarter_max(float v) {
+  float e, o;
+  row_swap(v, e, o);
+  return half_max(fmaxf(e, o));
+}
+__device__ __forceinline__ float quarter_sum(float v) {
+  float e, o;
+  row_swap(v, e, o);
+  return half_sum(e + o);
 }
 
 // Lazy-rescale threshold of the online softmax, in log2 units.

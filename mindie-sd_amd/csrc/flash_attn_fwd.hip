@@ -6,6 +6,10 @@
 // rainfusionattention (csrc/plugin/block_sparse_attention.cpp:31-121,
 // csrc/plugin/rainfusionattention.cpp:27-64).
 //
+// Two kernels share the algorithm: fa_fwd16_kernel (plain dense attention, 16x16x32 matrix instruction) and
+// fa_fwd_kernel (block-sparse, masked, causal and packed variable-length attention and the tuning variants of the
+// dense case, 32x32x16 instruction).  What follows describes fa_fwd_kernel; fa_fwd16_kernel states its differences.
+//
 // Algorithm: single pass, online softmax.  One workgroup owns BM = NWAVES*QPW query rows of one
 // (batch, head); it walks the key/value sequence in tiles of BN keys staged in LDS (double
 // buffered, one barrier per tile).  The kernel works on the TRANSPOSED problem so that every
@@ -587,6 +591,300 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// Dense attention on the 16x16x32 matrix instruction (8 waves x 32 query rows, 128-key tiles).  The same
+// transposed formulation as fa_fwd_kernel; what changes is the shape of the register tiles.  With c = lane % 16
+// and g = lane / 16:
+//     S^T block (16 keys x 16 queries):  A = K rows 16*kb + c, head_dim 32*ks + 8*g .. +8 (one 16-byte LDS read),
+//                                        B = Q^T resident (query 16*nq + c, same head_dim slice);
+//                                        the lane receives keys 16*kb + 4*g + i (i < 4) of query 16*nq + c
+//     O^T block (16 dims x 16 queries):  B = P^T of 32 keys straight from two S^T blocks (slot 8*g + t holds key
+//                                        32*j + 4*g + t for t < 4 and key 32*j + 16 + 4*g + t - 4 for t >= 4),
+//                                        A = V^T in the same slot order from two transposing LDS reads
+// A row maximum is 32 in-lane operations per tile and query column plus two lane exchanges (rows of 16 lanes, then
+// halves).  The instruction sustains 2.4 PFLOP/s where the 32x32x16 form stops at 2.1-2.2.
+// LDS: K stages at 0 and 32 KiB, V stages at 64 and 96 KiB, so that stage and row offsets of every read fit the
+// 16-bit offset field.  K rows are swizzled as in fa_fwd_kernel; V: 32-byte chunk c32 of row key is stored at chunk
+// c32 ^ (key & 7) - a half-wave of the transposing read covers 8 rows x 32 bytes.
+template <int DT>
+__global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using E = Elem<DT>;
+  using T = typename E::type;
+  using X8 = typename E::x8;
+  constexpr int NWAVES = 8, BN = 128, kBM = 256, kRowBytes = 256, kTileBytes = BN * kRowBytes;
+  constexpr int kORowBytes = kRowBytes + 8;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  MSD_LDS char* smem = (MSD_LDS char*)smem_raw;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15;
+  const int g = lane >> 4;
+
+  const int q_tiles = (p.Sq + kBM - 1) / kBM;
+  const int total = p.B * p.N * q_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
+  if (work >= total) return;
+  const int bn = work / q_tiles;
+  const int qt = work - bn * q_tiles;
+  const int b = bn / p.N;
+  const int n = bn - b * p.N;
+  const int nkv = n / (p.N / p.Nkv);
+  const int q0 = qt * kBM;
+  const int Sq = p.Sq, Skv = p.Skv;
+
+  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
+  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
+  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+
+  // ---- Q^T operand, resident: lane (c, g) holds query 16*nq + c, head_dim 32*ks + 8*g .. +8 --------------
+  X8 qf[2][4];
+#pragma unroll
+  for (int nq = 0; nq < 2; ++nq) {
+    const int qrow = q0 + wave * 32 + nq * 16 + c;
+    const bool ok = qrow < Sq;
+    const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      X8 v = *(const X8*)(src + 32 * ks);
+      if (!ok) v = X8{0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = E::from_float((float)v[j] * p.scale_log2);
+      qf[nq][ks] = v;
+    }
+  }
+
+  f32x4_t oacc[8][2];
+  float m_run[2], l_run[2];
+  f32x4_t negm[2];
+#pragma unroll
+  for (int nq = 0; nq < 2; ++nq) {
+    m_run[nq] = 0.f;
+    l_run[nq] = 0.f;
+    negm[nq] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int db = 0; db < 8; ++db) oacc[db][nq] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- global -> LDS staging (LDS-DMA; swizzles applied on the global side) -------------------------------
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)kg, 0, (int)(((long long)(Skv - 1) * p.k_ss + 128) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)vg, 0, (int)(((long long)(Skv - 1) * p.v_ss + 128) * 2), 0x00020000);
+  const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
+  int k_voff, v_voff;
+  {
+    const int row = 4 * wave + (lane >> 4);  // groups of one wave lie 32 rows apart: same swizzles
+    const int pc = lane & 15;                // physical 16-byte chunk this lane fills
+    k_voff = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
+    v_voff = row * v_row_bytes + (((((pc >> 1) ^ (row & 7)) << 1) | (pc & 1)) << 4);
+  }
+  auto load_tile = [&](int key0, int stage) {
+    tile_dma<BN / 4 / NWAVES, NWAVES>(k_rsrc, v_rsrc, smem + stage * kTileBytes, smem + (2 + stage) * kTileBytes, k_voff,
+                                      v_voff, wave, key0 * k_row_bytes, key0 * v_row_bytes, k_row_bytes, v_row_bytes);
+  };
+
+  // per-lane parts of the LDS read addresses
+  // K operand: row 16*kb + c, 16-byte chunk (4*ks + g) ^ c
+  unsigned k_lds[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) k_lds[ks] = (unsigned)(uintptr_t)smem + c * kRowBytes + (((4 * ks + g) ^ c) << 4);
+  // V^T operand: the lane points at key 4*g + c/4 (+32*j, +16), 8 bytes at 8*(c%4) of 32-byte chunk db ^ (key & 7)
+  // (blocks db and db + 4 differ in bit 7 of the address only: four registers, the other four by one XOR)
+  unsigned v_lds[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+    v_lds[db] = (unsigned)(uintptr_t)smem + 2 * kTileBytes + (4 * g + (c >> 2)) * kRowBytes +
+                ((db ^ (4 * (g & 1) + (c >> 2))) << 5) + 8 * (c & 3);
+
+  const int tiles = (Skv + BN - 1) / BN;
+  load_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  bool first = true;
+
+  auto tile_step = [&](auto stage_c, const int key0, const int next_key0) {
+    constexpr int stage = decltype(stage_c)::value;
+    if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+
+    // ---- S^T = K Q^T: 16 accumulation chains; operand reads in groups of 2 key blocks of one 32-wide head_dim
+    // step, two groups ahead of the matrix instructions that use them (ring of three) ---------------------------
+    f32x4_t sacc[8][2];
+    X8 afrag[3][2];
+    auto k_read = [&](auto gi_c, X8(&dst)[2]) __attribute__((always_inline)) {
+      constexpr int gi = decltype(gi_c)::value;
+      constexpr int ks = gi >> 2, qu = gi & 3;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        dst[i] = *(MSD_LDS const X8*)(uintptr_t)(k_lds[ks] + stage * kTileBytes + (2 * qu + i) * 16 * kRowBytes);
+    };
+    k_read(std::integral_constant<int, 0>{}, afrag[0]);
+    k_read(std::integral_constant<int, 1>{}, afrag[1]);
+    static_for<16>([&](auto gi_c) __attribute__((always_inline)) {
+      constexpr int gi = decltype(gi_c)::value;
+      constexpr int ks = gi >> 2, qu = gi & 3;
+      if constexpr (gi + 2 < 16) k_read(std::integral_constant<int, gi + 2>{}, afrag[(gi + 2) % 3]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int nq = 0; nq < 2; ++nq)
+          sacc[2 * qu + i][nq] =
+              E::mfma16(afrag[gi % 3][i], qf[nq][ks], ks == 0 ? negm[nq] : sacc[2 * qu + i][nq]);
+    });
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int gi = 0; gi < 14; ++gi) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- keys past the end of the sequence (last tile only) ---------------------------------------------------
+    if (key0 + BN > Skv) {
+#pragma unroll
+      for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + 16 * kb + 4 * g + i >= Skv) {
+            sacc[kb][0][i] = -INFINITY;
+            sacc[kb][1][i] = -INFINITY;
+          }
+    }
+
+    // ---- online softmax (exp2 domain, lazily moved reference maximum; see fa_fwd_kernel) ---------------------
+    X8 pf[2][4];
+#pragma unroll
+    for (int nq = 0; nq < 2; ++nq) {
+      float mx = sacc[0][nq][0];
+#pragma unroll
+      for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
+      mx = quarter_max(mx);
+      if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+        float delta = first ? mx : fmaxf(mx, 0.f);
+        delta = (delta == -INFINITY) ? 0.f : delta;
+        const float alpha = fast_exp2(-delta);
+        m_run[nq] += delta;
+        l_run[nq] *= alpha;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) negm[nq][i] = -m_run[nq];
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sacc[kb][nq][i] -= delta;
+#pragma unroll
+        for (int db = 0; db < 8; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[db][nq][i] *= alpha;
+      }
+      float ls = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        X8 pk;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          pk[t] = E::from_float(fast_exp2(sacc[2 * j][nq][t]));
+          pk[4 + t] = E::from_float(fast_exp2(sacc[2 * j + 1][nq][t]));
+        }
+        pf[nq][j] = pk;
+        ls = E::sum8(pk, ls);
+      }
+      l_run[nq] += ls;
+    }
+
+    // ---- O^T += V^T P^T: 8 steps of (32 keys) x (4 head_dim blocks); V^T fragments requested one step ahead
+    // with asm reads and explicit waits, so that the next tile's LDS-DMA stays in flight (see lds_read_tr16_async)
+    s16x4_t vf[2][8];
+    auto issue = [&](auto step_c, s16x4_t(&dst)[8]) __attribute__((always_inline)) {
+      constexpr int s = decltype(step_c)::value;
+      constexpr int j = s >> 1, dbh = s & 1;
+      constexpr int off = stage * kTileBytes + 32 * j * kRowBytes;
+#pragma unroll
+      for (int d4 = 0; d4 < 4; ++d4) {
+        const unsigned a = v_lds[d4] ^ (dbh << 7);
+        dst[2 * d4] = lds_read_tr16_async<off>(a);
+        dst[2 * d4 + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(a);
+      }
+    };
+    issue(std::integral_constant<int, 0>{}, vf[0]);
+    static_for<8>([&](auto step_c) __attribute__((always_inline)) {
+      constexpr int s = decltype(step_c)::value;
+      constexpr int j = s >> 1, dbh = s & 1;
+      if constexpr (s + 1 < 8) {
+        issue(std::integral_constant<int, s + 1>{}, vf[(s + 1) & 1]);
+        lds_wait_tr<8>(vf[s & 1]);
+      } else {
+        lds_wait_tr<0>(vf[s & 1]);
+      }
+#pragma unroll
+      for (int d4 = 0; d4 < 4; ++d4) {
+        union { s16x4_t s2[2]; X8 x; } u;
+        u.s2[0] = vf[s & 1][2 * d4];
+        u.s2[1] = vf[s & 1][2 * d4 + 1];
+#pragma unroll
+        for (int nq = 0; nq < 2; ++nq) oacc[4 * dbh + d4][nq] = E::mfma16(u.x, pf[nq][j], oacc[4 * dbh + d4][nq]);
+      }
+    });
+
+    first = false;
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next tile has landed
+    __syncthreads();
+  };
+  for (int t = 0; t < tiles; t += 2) {
+    tile_step(std::integral_constant<int, 0>{}, t * BN, t + 1 < tiles ? (t + 1) * BN : -1);
+    if (t + 1 < tiles) tile_step(std::integral_constant<int, 1>{}, (t + 1) * BN, t + 2 < tiles ? (t + 2) * BN : -1);
+  }
+
+  // ---- epilogue: normalise, transpose the wave's 32 query rows through LDS, coalesced store --------------------
+  MSD_LDS char* ost = smem + wave * 32 * kORowBytes;
+#pragma unroll
+  for (int nq = 0; nq < 2; ++nq) {
+    const float l_tot = quarter_sum(l_run[nq]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int qrow_l = q0 + wave * 32 + nq * 16 + c;
+    if (p.lse && g == 0 && qrow_l < Sq)
+      p.lse[((long long)b * p.N + n) * p.Sq + qrow_l] =
+          l_tot > 0.f ? m_run[nq] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      typename E::x4 pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pk[i] = E::from_float(oacc[db][nq][i] * inv);
+      *(MSD_LDS typename E::x4*)(ost + (nq * 16 + c) * kORowBytes + (16 * db + 4 * g) * 2) = pk;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int i = 0; i < 32 * 16 / 64; ++i) {
+    const int ch = i * 64 + lane;
+    const int row = ch >> 4, c16 = ch & 15;
+    const int qrow = q0 + wave * 32 + row;
+    const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16);
+    const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16 + 8);
+    if (qrow < Sq) {
+      i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
+      *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = v;
+    }
+  }
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+template <int DT>
+static int launch_fa16(const FaParams& p, hipStream_t stream) {
+  constexpr int kLds = 4 * 128 * 256;  // two K and two V stages of 128 keys
+  auto kern = fa_fwd16_kernel<DT>;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+    return MSD_ERR_LAUNCH;
+  const int total = p.B * p.N * ((p.Sq + 255) / 256);
+  hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(512), kLds, stream, p);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -608,8 +906,9 @@ using namespace msd;
 extern "C" {
 
 // Tuning hook used by benchmark sweeps: selects the dense kernel variant
-// (0, default: 8 waves x 32 rows, 128-key tiles, operand reads scheduled one step ahead;
-//  1: 4 waves x 32 rows, 64-key tiles, compiler scheduling; 2: as 0 with compiler scheduling;
+// (0, default: fa_fwd16_kernel, 8 waves x 32 rows, 128-key tiles on the 16x16x32 matrix instruction;
+//  4: the same tile shape on the 32x32x16 instruction (fa_fwd_kernel), operand reads scheduled one step ahead;
+//  1: 4 waves x 32 rows, 64-key tiles, compiler scheduling; 2: as 4 with compiler scheduling;
 //  3: as 1 with scheduled operand reads).
 static int g_dense_variant = 0;
 static int g_map_mode = 0;  // bits 8.. of the variant: tile order (0 = per-XCD chunks, 1 = linear)
@@ -712,10 +1011,11 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
       case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);
       case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
       case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);
-      default: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1>(p, stream);
+      case 4: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1>(p, stream);
+      default: return launch_fa16<MSD_DTYPE_BF16>(p, stream);
     }
   }
-  return launch_fa<MSD_DTYPE_F16, 8, 32, 128, false, 1>(p, stream);
+  return launch_fa16<MSD_DTYPE_F16>(p, stream);
 }
 
 // Block-sparse attention with an optional causal mask inside the selected blocks (queries and keys of equal
