@@ -29,6 +29,10 @@
 
 #include "common.hpp"
 
+#ifndef FA16_AHEAD
+#define FA16_AHEAD 3  // K operand groups requested ahead of their use in fa_fwd16_kernel
+#endif
+
 namespace msd {
 
 struct FaParams {
@@ -429,8 +433,9 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][qb][r]);
-      mx = half_max(mx);
+      // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
       if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+        mx = half_max(mx);
         // first tile: move to the exact row maximum (delta may be negative); later: only upwards
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
@@ -605,13 +610,13 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 // LDS: K stages at 0 and 32 KiB, V stages at 64 and 96 KiB, so that stage and row offsets of every read fit the
 // 16-bit offset field.  K rows are swizzled as in fa_fwd_kernel; V: 32-byte chunk c32 of row key is stored at chunk
 // c32 ^ (key & 7) - a half-wave of the transposing read covers 8 rows x 32 bytes.
-template <int DT>
-__global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
+template <int DT, int NWAVES = 8>
+__global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
   using T = typename E::type;
   using X8 = typename E::x8;
-  constexpr int NWAVES = 8, BN = 128, kBM = 256, kRowBytes = 256, kTileBytes = BN * kRowBytes;
+  constexpr int BN = 128, kBM = NWAVES * 32, kRowBytes = 256, kTileBytes = BN * kRowBytes;
   constexpr int kORowBytes = kRowBytes + 8;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   MSD_LDS char* smem = (MSD_LDS char*)smem_raw;
@@ -677,7 +682,7 @@ __global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
   int k_voff, v_voff;
   {
-    const int row = 4 * wave + (lane >> 4);  // groups of one wave lie 32 rows apart: same swizzles
+    const int row = 4 * wave + (lane >> 4);  // groups of one wave lie 4 * NWAVES rows apart: same swizzles
     const int pc = lane & 15;                // physical 16-byte chunk this lane fills
     k_voff = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
     v_voff = row * v_row_bytes + (((((pc >> 1) ^ (row & 7)) << 1) | (pc & 1)) << 4);
@@ -711,9 +716,10 @@ __global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
 
     // ---- S^T = K Q^T: 16 accumulation chains; operand reads in groups of 2 key blocks of one 32-wide head_dim
-    // step, two groups ahead of the matrix instructions that use them (ring of three) ---------------------------
+    // step, kAhead groups ahead of the matrix instructions that use them (ring of kAhead + 1) -----------------
     f32x4_t sacc[8][2];
-    X8 afrag[3][2];
+    constexpr int kAhead = FA16_AHEAD;
+    X8 afrag[kAhead + 1][2];
     auto k_read = [&](auto gi_c, X8(&dst)[2]) __attribute__((always_inline)) {
       constexpr int gi = decltype(gi_c)::value;
       constexpr int ks = gi >> 2, qu = gi & 3;
@@ -721,26 +727,25 @@ __global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
       for (int i = 0; i < 2; ++i)
         dst[i] = *(MSD_LDS const X8*)(uintptr_t)(k_lds[ks] + stage * kTileBytes + (2 * qu + i) * 16 * kRowBytes);
     };
-    k_read(std::integral_constant<int, 0>{}, afrag[0]);
-    k_read(std::integral_constant<int, 1>{}, afrag[1]);
+    static_for<kAhead>([&](auto gi_c) __attribute__((always_inline)) { k_read(gi_c, afrag[decltype(gi_c)::value]); });
     static_for<16>([&](auto gi_c) __attribute__((always_inline)) {
       constexpr int gi = decltype(gi_c)::value;
       constexpr int ks = gi >> 2, qu = gi & 3;
-      if constexpr (gi + 2 < 16) k_read(std::integral_constant<int, gi + 2>{}, afrag[(gi + 2) % 3]);
+      if constexpr (gi + kAhead < 16) k_read(std::integral_constant<int, gi + kAhead>{}, afrag[(gi + kAhead) % (kAhead + 1)]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int nq = 0; nq < 2; ++nq)
           sacc[2 * qu + i][nq] =
-              E::mfma16(afrag[gi % 3][i], qf[nq][ks], ks == 0 ? negm[nq] : sacc[2 * qu + i][nq]);
+              E::mfma16(afrag[gi % (kAhead + 1)][i], qf[nq][ks], ks == 0 ? negm[nq] : sacc[2 * qu + i][nq]);
     });
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
 #pragma unroll
-    for (int gi = 0; gi < 14; ++gi) {
+    for (int gi = 0; gi < 16 - kAhead; ++gi) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- keys past the end of the sequence (last tile only) ---------------------------------------------------
@@ -764,8 +769,9 @@ __global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
       for (int kb = 0; kb < 8; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
-      mx = quarter_max(mx);
+      // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
       if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+        mx = quarter_max(mx);
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
         const float alpha = fast_exp2(-delta);
@@ -874,14 +880,14 @@ __global__ __launch_bounds__(512, 1) void fa_fwd16_kernel(const FaParams p) {
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT>
+template <int DT, int NWAVES = 8>
 static int launch_fa16(const FaParams& p, hipStream_t stream) {
   constexpr int kLds = 4 * 128 * 256;  // two K and two V stages of 128 keys
-  auto kern = fa_fwd16_kernel<DT>;
+  auto kern = fa_fwd16_kernel<DT, NWAVES>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const int total = p.B * p.N * ((p.Sq + 255) / 256);
-  hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(512), kLds, stream, p);
+  const int total = p.B * p.N * ((p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
+  hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
@@ -1012,6 +1018,7 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
       case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
       case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);
       case 4: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1>(p, stream);
+      case 5: return launch_fa16<MSD_DTYPE_BF16, 4>(p, stream);
       default: return launch_fa16<MSD_DTYPE_BF16>(p, stream);
     }
   }

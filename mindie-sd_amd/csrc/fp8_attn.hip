@@ -507,8 +507,10 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     i32x8_t pf[2];
     if (P2) {
       // sacc = s - m_run + kPShift; the reference maximum moves when a row exceeds it by more than kTau8
-      mx = half_max(mx) - kPShift;
+      // (tested on the lanes' own parts: one of them exceeds the threshold iff a row maximum does)
+      mx -= kPShift;
       if (first || __builtin_amdgcn_ballot_w64(mx > kTau8) != 0) {
+        mx = half_max(mx);
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
         const float alpha = fast_exp2(-delta);
@@ -536,8 +538,9 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
                                  fast_exp2(sacc[kb][4 * g4 + 2]), fast_exp2(sacc[kb][4 * g4 + 3]));
       }
     } else {
-    mx = half_max(mx) * c;
+    mx *= c;
     if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau8) != 0) {
+      mx = half_max(mx);
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
       m_run = m_new;
