@@ -30,7 +30,7 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes of one dense 14B-720p launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by a 1 GiB copy kernel (summary and commands: profiles/fa_fwd_dense_bf16_wan14b_720p.md)
-DENSE_TRAFFIC_BYTES = 1.70e10
+DENSE_TRAFFIC_BYTES = 1.72e10
 
 # workloads
 CFG_14B_720P = dict(B=1, N=40, S=75600, D=128, grid=(21, 45, 80))
@@ -388,7 +388,7 @@ def main():
         "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": DENSE_TRAFFIC_BYTES,
-                     "kernel": "fa_fwd_kernel<bf16, 8 waves x 32 rows, 128-key tiles>",
+                     "kernel": "fa_fwd16_kernel<bf16, 8 waves x 32 rows, 128-key tiles>",
                      "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms},
     }
     if not args.no_extras:

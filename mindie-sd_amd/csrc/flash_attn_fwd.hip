@@ -663,11 +663,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   }
 
   f32x4_t oacc[8][2];
-  float m_run[2], l_run[2];
-  f32x4_t negm[2];
+  float l_run[2];
+  f32x4_t negm[2];  // minus the reference maximum (log2 units), in the four slots that seed an accumulator
 #pragma unroll
   for (int nq = 0; nq < 2; ++nq) {
-    m_run[nq] = 0.f;
     l_run[nq] = 0.f;
     negm[nq] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -775,10 +774,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
         const float alpha = fast_exp2(-delta);
-        m_run[nq] += delta;
+        const float nm = negm[nq][0] - delta;
         l_run[nq] *= alpha;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) negm[nq][i] = -m_run[nq];
+        for (int i = 0; i < 4; ++i) negm[nq][i] = nm;
 #pragma unroll
         for (int kb = 0; kb < 8; ++kb)
 #pragma unroll
@@ -855,7 +854,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     const int qrow_l = q0 + wave * 32 + nq * 16 + c;
     if (p.lse && g == 0 && qrow_l < Sq)
       p.lse[((long long)b * p.N + n) * p.Sq + qrow_l] =
-          l_tot > 0.f ? m_run[nq] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
+          l_tot > 0.f ? -negm[nq][0] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
       typename E::x4 pk;
