@@ -30,7 +30,7 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes of one dense 14B-720p launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by a 1 GiB copy kernel (summary and commands: profiles/fa_fwd_dense_bf16_wan14b_720p.md)
-DENSE_TRAFFIC_BYTES = 1.72e10
+DENSE_TRAFFIC_BYTES = 1.71e10
 
 # workloads
 CFG_14B_720P = dict(B=1, N=40, S=75600, D=128, grid=(21, 45, 80))
