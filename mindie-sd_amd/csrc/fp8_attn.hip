@@ -35,7 +35,8 @@ __device__ __forceinline__ int pack4_e4m3(float a, float b, float c, float d) {
 }
 // probabilities are already inside the range: no clamp
 __device__ __forceinline__ int pack4_e4m3_noclamp(float a, float b, float c, float d) {
-  int w = 0;
+  int w;
+  asm volatile("" : "=v"(w));  // any register content: both halves are overwritten (saves the move zero would cost)
   w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
   w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
   return w;
