@@ -154,6 +154,98 @@ __device__ __forceinline__ float quarter_sum(float v) {
   return half_sum(e + o);
 }
 
+// Rescale of one 16-query column block of fa_fwd16_kernel when its reference maximum moves: l *= alpha, the seed and
+// the 8 score blocks -= delta, the 8 output blocks *= alpha - 69 registers updated in place by three asm blocks, each
+// skipped by its own branch when the wave-uniform flag is zero.  The test and the branches sit inside the asm, so the
+// compiler sees straight-line code that leaves every value in its register.  Written as an if/else in C++, the rarely
+// taken update lands in other registers and the path that skips it pays some 100 register moves per tile to meet it
+// at the join.  (None of the values may be the result of a matrix instruction still in flight: the compiler cannot
+// place the wait states such a read needs inside an asm block.  Here the scores have been read by the maximum and
+// the outputs were written a whole phase earlier.)
+__device__ __forceinline__ void cond_rescale_fa16(int flag, float delta, float alpha, float& l, f32x4_t& negm, f32x4_t& s0,
+                                                  f32x4_t& s1, f32x4_t& s2, f32x4_t& s3, f32x4_t& s4, f32x4_t& s5,
+                                                  f32x4_t& s6, f32x4_t& s7, f32x4_t& o0, f32x4_t& o1, f32x4_t& o2,
+                                                  f32x4_t& o3, f32x4_t& o4, f32x4_t& o5, f32x4_t& o6, f32x4_t& o7) {
+  float negm_0 = negm[0], negm_1 = negm[1], negm_2 = negm[2], negm_3 = negm[3];
+  float s0_0 = s0[0], s0_1 = s0[1], s0_2 = s0[2], s0_3 = s0[3];
+  float s1_0 = s1[0], s1_1 = s1[1], s1_2 = s1[2], s1_3 = s1[3];
+  float s2_0 = s2[0], s2_1 = s2[1], s2_2 = s2[2], s2_3 = s2[3];
+  float s3_0 = s3[0], s3_1 = s3[1], s3_2 = s3[2], s3_3 = s3[3];
+  float s4_0 = s4[0], s4_1 = s4[1], s4_2 = s4[2], s4_3 = s4[3];
+  float s5_0 = s5[0], s5_1 = s5[1], s5_2 = s5[2], s5_3 = s5[3];
+  float s6_0 = s6[0], s6_1 = s6[1], s6_2 = s6[2], s6_3 = s6[3];
+  float s7_0 = s7[0], s7_1 = s7[1], s7_2 = s7[2], s7_3 = s7[3];
+  float o0_0 = o0[0], o0_1 = o0[1], o0_2 = o0[2], o0_3 = o0[3];
+  float o1_0 = o1[0], o1_1 = o1[1], o1_2 = o1[2], o1_3 = o1[3];
+  float o2_0 = o2[0], o2_1 = o2[1], o2_2 = o2[2], o2_3 = o2[3];
+  float o3_0 = o3[0], o3_1 = o3[1], o3_2 = o3[2], o3_3 = o3[3];
+  float o4_0 = o4[0], o4_1 = o4[1], o4_2 = o4[2], o4_3 = o4[3];
+  float o5_0 = o5[0], o5_1 = o5[1], o5_2 = o5[2], o5_3 = o5[3];
+  float o6_0 = o6[0], o6_1 = o6[1], o6_2 = o6[2], o6_3 = o6[3];
+  float o7_0 = o7[0], o7_1 = o7[1], o7_2 = o7[2], o7_3 = o7[3];
+  asm volatile("s_cmp_eq_u32 %25, 0\n\t" "s_cbranch_scc1 .Lmsd_skip%=\n\t" "v_mul_f32 %0, %0, %27\n\t"
+               "v_sub_f32 %1, %1, %26\n\t" "v_sub_f32 %2, %2, %26\n\t" "v_sub_f32 %3, %3, %26\n\t"
+               "v_sub_f32 %4, %4, %26\n\t" "v_sub_f32 %5, %5, %26\n\t" "v_sub_f32 %6, %6, %26\n\t"
+               "v_sub_f32 %7, %7, %26\n\t" "v_sub_f32 %8, %8, %26\n\t" "v_sub_f32 %9, %9, %26\n\t"
+               "v_sub_f32 %10, %10, %26\n\t" "v_sub_f32 %11, %11, %26\n\t" "v_sub_f32 %12, %12, %26\n\t"
+               "v_sub_f32 %13, %13, %26\n\t" "v_sub_f32 %14, %14, %26\n\t" "v_sub_f32 %15, %15, %26\n\t"
+               "v_sub_f32 %16, %16, %26\n\t" "v_sub_f32 %17, %17, %26\n\t" "v_sub_f32 %18, %18, %26\n\t"
+               "v_sub_f32 %19, %19, %26\n\t" "v_sub_f32 %20, %20, %26\n\t" "v_sub_f32 %21, %21, %26\n\t"
+               "v_sub_f32 %22, %22, %26\n\t" "v_sub_f32 %23, %23, %26\n\t" "v_sub_f32 %24, %24, %26\n\t"
+               "s_nop 7\n\t" ".Lmsd_skip%=:"
+               : "+v"(l), "+v"(negm_0), "+v"(negm_1), "+v"(negm_2), "+v"(negm_3), "+v"(s0_0), "+v"(s0_1), "+v"(s0_2),
+                 "+v"(s0_3), "+v"(s1_0), "+v"(s1_1), "+v"(s1_2), "+v"(s1_3), "+v"(s2_0), "+v"(s2_1), "+v"(s2_2),
+                 "+v"(s2_3), "+v"(s3_0), "+v"(s3_1), "+v"(s3_2), "+v"(s3_3), "+v"(s4_0), "+v"(s4_1), "+v"(s4_2),
+                 "+v"(s4_3)
+               : "s"(flag), "v"(delta), "v"(alpha)
+               : "scc");
+  asm volatile("s_cmp_eq_u32 %24, 0\n\t" "s_cbranch_scc1 .Lmsd_skip%=\n\t" "v_sub_f32 %0, %0, %25\n\t"
+               "v_sub_f32 %1, %1, %25\n\t" "v_sub_f32 %2, %2, %25\n\t" "v_sub_f32 %3, %3, %25\n\t"
+               "v_sub_f32 %4, %4, %25\n\t" "v_sub_f32 %5, %5, %25\n\t" "v_sub_f32 %6, %6, %25\n\t"
+               "v_sub_f32 %7, %7, %25\n\t" "v_sub_f32 %8, %8, %25\n\t" "v_sub_f32 %9, %9, %25\n\t"
+               "v_sub_f32 %10, %10, %25\n\t" "v_sub_f32 %11, %11, %25\n\t" "v_mul_f32 %12, %12, %26\n\t"
+               "v_mul_f32 %13, %13, %26\n\t" "v_mul_f32 %14, %14, %26\n\t" "v_mul_f32 %15, %15, %26\n\t"
+               "v_mul_f32 %16, %16, %26\n\t" "v_mul_f32 %17, %17, %26\n\t" "v_mul_f32 %18, %18, %26\n\t"
+               "v_mul_f32 %19, %19, %26\n\t" "v_mul_f32 %20, %20, %26\n\t" "v_mul_f32 %21, %21, %26\n\t"
+               "v_mul_f32 %22, %22, %26\n\t" "v_mul_f32 %23, %23, %26\n\t" "s_nop 7\n\t"
+               ".Lmsd_skip%=:"
+               : "+v"(s5_0), "+v"(s5_1), "+v"(s5_2), "+v"(s5_3), "+v"(s6_0), "+v"(s6_1), "+v"(s6_2), "+v"(s6_3),
+                 "+v"(s7_0), "+v"(s7_1), "+v"(s7_2), "+v"(s7_3), "+v"(o0_0), "+v"(o0_1), "+v"(o0_2), "+v"(o0_3),
+                 "+v"(o1_0), "+v"(o1_1), "+v"(o1_2), "+v"(o1_3), "+v"(o2_0), "+v"(o2_1), "+v"(o2_2), "+v"(o2_3)
+               : "s"(flag), "v"(delta), "v"(alpha)
+               : "scc");
+  asm volatile("s_cmp_eq_u32 %20, 0\n\t" "s_cbranch_scc1 .Lmsd_skip%=\n\t" "v_mul_f32 %0, %0, %21\n\t"
+               "v_mul_f32 %1, %1, %21\n\t" "v_mul_f32 %2, %2, %21\n\t" "v_mul_f32 %3, %3, %21\n\t"
+               "v_mul_f32 %4, %4, %21\n\t" "v_mul_f32 %5, %5, %21\n\t" "v_mul_f32 %6, %6, %21\n\t"
+               "v_mul_f32 %7, %7, %21\n\t" "v_mul_f32 %8, %8, %21\n\t" "v_mul_f32 %9, %9, %21\n\t"
+               "v_mul_f32 %10, %10, %21\n\t" "v_mul_f32 %11, %11, %21\n\t" "v_mul_f32 %12, %12, %21\n\t"
+               "v_mul_f32 %13, %13, %21\n\t" "v_mul_f32 %14, %14, %21\n\t" "v_mul_f32 %15, %15, %21\n\t"
+               "v_mul_f32 %16, %16, %21\n\t" "v_mul_f32 %17, %17, %21\n\t" "v_mul_f32 %18, %18, %21\n\t"
+               "v_mul_f32 %19, %19, %21\n\t" "s_nop 7\n\t" ".Lmsd_skip%=:"
+               : "+v"(o3_0), "+v"(o3_1), "+v"(o3_2), "+v"(o3_3), "+v"(o4_0), "+v"(o4_1), "+v"(o4_2), "+v"(o4_3),
+                 "+v"(o5_0), "+v"(o5_1), "+v"(o5_2), "+v"(o5_3), "+v"(o6_0), "+v"(o6_1), "+v"(o6_2), "+v"(o6_3),
+                 "+v"(o7_0), "+v"(o7_1), "+v"(o7_2), "+v"(o7_3)
+               : "s"(flag), "v"(alpha)
+               : "scc");
+  negm = f32x4_t{negm_0, negm_1, negm_2, negm_3};
+  s0 = f32x4_t{s0_0, s0_1, s0_2, s0_3};
+  s1 = f32x4_t{s1_0, s1_1, s1_2, s1_3};
+  s2 = f32x4_t{s2_0, s2_1, s2_2, s2_3};
+  s3 = f32x4_t{s3_0, s3_1, s3_2, s3_3};
+  s4 = f32x4_t{s4_0, s4_1, s4_2, s4_3};
+  s5 = f32x4_t{s5_0, s5_1, s5_2, s5_3};
+  s6 = f32x4_t{s6_0, s6_1, s6_2, s6_3};
+  s7 = f32x4_t{s7_0, s7_1, s7_2, s7_3};
+  o0 = f32x4_t{o0_0, o0_1, o0_2, o0_3};
+  o1 = f32x4_t{o1_0, o1_1, o1_2, o1_3};
+  o2 = f32x4_t{o2_0, o2_1, o2_2, o2_3};
+  o3 = f32x4_t{o3_0, o3_1, o3_2, o3_3};
+  o4 = f32x4_t{o4_0, o4_1, o4_2, o4_3};
+  o5 = f32x4_t{o5_0, o5_1, o5_2, o5_3};
+  o6 = f32x4_t{o6_0, o6_1, o6_2, o6_3};
+  o7 = f32x4_t{o7_0, o7_1, o7_2, o7_3};
+}
+
 // Lazy-rescale threshold of the online softmax, in log2 units.
 constexpr float kTau = 8.0f;
 

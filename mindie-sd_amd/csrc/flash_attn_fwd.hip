@@ -769,24 +769,19 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
       // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
+      float delta = 0.f, alpha = 1.f;
+      int moved = 0;
       if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
         mx = quarter_max(mx);
-        float delta = first ? mx : fmaxf(mx, 0.f);
+        delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
-        const float alpha = fast_exp2(-delta);
-        const float nm = negm[nq][0] - delta;
-        l_run[nq] *= alpha;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) negm[nq][i] = nm;
-#pragma unroll
-        for (int kb = 0; kb < 8; ++kb)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) sacc[kb][nq][i] -= delta;
-#pragma unroll
-        for (int db = 0; db < 8; ++db)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) oacc[db][nq][i] *= alpha;
+        alpha = fast_exp2(-delta);
+        moved = 1;
       }
+      // the rescale itself: in place, skipped when the reference did not move (see cond_rescale_fa16)
+      cond_rescale_fa16(__builtin_amdgcn_readfirstlane(moved), delta, alpha, l_run[nq], negm[nq], sacc[0][nq], sacc[1][nq],
+                        sacc[2][nq], sacc[3][nq], sacc[4][nq], sacc[5][nq], sacc[6][nq], sacc[7][nq], oacc[0][nq],
+                        oacc[1][nq], oacc[2][nq], oacc[3][nq], oacc[4][nq], oacc[5][nq], oacc[6][nq], oacc[7][nq]);
       float ls = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
