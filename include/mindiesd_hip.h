@@ -210,6 +210,17 @@ int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, in
                          long long v_sb, long long v_sn, long long v_ss, void* workspace, size_t ws_bytes,
                          hipStream_t stream);
 
+/* mindiesd_fp8_v_quant for callers that cannot allocate (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same inputs, outputs and results,
+ * no workspace argument: the per-channel maxima live in a fixed device array inside the library (2 MiB per GPU,
+ * held until the process ends), which limits B * N to mindiesd_fp8_v_quant_static_max_heads() = 4096 (beyond
+ * that: return code 3).  Nothing is allocated or freed, no stream is synchronised.  All calls on one GPU share
+ * that array: calls that overlap on one GPU (different streams or threads) race and must be serialised by the
+ * caller. */
+int mindiesd_fp8_v_quant_static_max_heads(void);
+int mindiesd_fp8_v_quant_static(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
+                                long long v_sb, long long v_sn, long long v_ss, hipStream_t stream);
+
 /* FP8 flash attention on operands produced by the two functions above (Q/K with block_size 128).
  * Replaces torch_npu.npu_fused_infer_attention_score_v2 with per-block dequantisation scales as
  * called by FP8RotateQuantFA.forward (mindiesd/quantization/layer.py:304-316).

@@ -16,13 +16,18 @@
 //            group of 64 keys the keys are stored in the order in which the S^T accumulator of the
 //            first product hands them to the second one: position 32*h + j holds key
 //            32*(j/16) + 8*((j%16)/4) + 4*h + j%4   (h = 0,1 the wave half, j = 0..31).
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
 
+// (batch x head) pairs that mindiesd_fp8_v_quant_static accepts: its scratch is a fixed device array
+#define MINDIESD_FP8_V_QUANT_STATIC_MAX_HEADS 4096
+
 namespace msd {
 
 constexpr float kE4M3Max = 448.0f;
+constexpr int kMaxDevices = 64;  // device ordinals the per-device scratch table covers
 
 __device__ __forceinline__ float clamp448(float x) { return __builtin_amdgcn_fmed3f(x, -kE4M3Max, kE4M3Max); }
 
@@ -673,31 +678,74 @@ int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float
 // bytes of the caller-provided scratch for mindiesd_fp8_v_quant (per-channel maxima)
 size_t mindiesd_fp8_v_quant_workspace_size(int B, int N) { return (size_t)B * N * 128 * sizeof(unsigned); }
 
-int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
-                         long long v_sb, long long v_sn, long long v_ss, void* workspace, size_t ws_bytes,
-                         hipStream_t stream) {
-  if (!v || !v8t || !v_scale || !workspace || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
-  if (D != 128) return MSD_ERR_UNSUPPORTED;
-  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
-  if (ws_bytes < mindiesd_fp8_v_quant_workspace_size(B, N)) return MSD_ERR_WORKSPACE;
-  if (((uintptr_t)v & 15) || ((uintptr_t)v8t & 15) || ((v_sb | v_sn | v_ss) & 7)) return MSD_ERR_BAD_ARG;
+// The three launches of the V quantisation; amax is scratch of B * N * 128 words that the first launch clears.
+static int v_quant_launch(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, long long v_sb,
+                          long long v_sn, long long v_ss, unsigned* amax, hipStream_t stream) {
   const long long nbits = (long long)B * N * 128;
   const int S128 = (S + 127) / 128 * 128;
-  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nbits + 255) / 256)), dim3(256), 0, stream, (unsigned*)workspace,
-                     0u, nbits);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nbits + 255) / 256)), dim3(256), 0, stream, amax, 0u, nbits);
   dim3 g1((S + 1023) / 1024, B * N), g2(S128 / 128, B * N);
   if (dtype == MSD_DTYPE_BF16) {
-    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_BF16>, g1, dim3(256), 0, stream, v, (unsigned*)workspace, v_sb, v_sn,
-                       v_ss, N, S);
-    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_BF16>, g2, dim3(256), 0, stream, v,
-                       (const unsigned*)workspace, (unsigned char*)v8t, v_scale, v_sb, v_sn, v_ss, N, S, S128);
+    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_BF16>, g1, dim3(256), 0, stream, v, amax, v_sb, v_sn, v_ss, N, S);
+    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_BF16>, g2, dim3(256), 0, stream, v, (const unsigned*)amax,
+                       (unsigned char*)v8t, v_scale, v_sb, v_sn, v_ss, N, S, S128);
   } else {
-    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_F16>, g1, dim3(256), 0, stream, v, (unsigned*)workspace, v_sb, v_sn,
-                       v_ss, N, S);
-    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_F16>, g2, dim3(256), 0, stream, v, (const unsigned*)workspace,
+    hipLaunchKernelGGL(channel_amax_kernel<MSD_DTYPE_F16>, g1, dim3(256), 0, stream, v, amax, v_sb, v_sn, v_ss, N, S);
+    hipLaunchKernelGGL(v_quant_transpose_kernel<MSD_DTYPE_F16>, g2, dim3(256), 0, stream, v, (const unsigned*)amax,
                        (unsigned char*)v8t, v_scale, v_sb, v_sn, v_ss, N, S, S128);
   }
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+static int v_quant_check(const void* v, const void* v8t, const float* v_scale, int dtype, int B, int N, int S, int D,
+                         long long v_sb, long long v_sn, long long v_ss) {
+  if (!v || !v8t || !v_scale || B <= 0 || N <= 0 || S <= 0) return MSD_ERR_BAD_ARG;
+  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if (((uintptr_t)v & 15) || ((uintptr_t)v8t & 15) || ((v_sb | v_sn | v_ss) & 7)) return MSD_ERR_BAD_ARG;
+  if ((long long)B * N > 65535) return MSD_ERR_UNSUPPORTED;  // grid.y
+  return MSD_OK;
+}
+
+int mindiesd_fp8_v_quant(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
+                         long long v_sb, long long v_sn, long long v_ss, void* workspace, size_t ws_bytes,
+                         hipStream_t stream) {
+  const int rc = v_quant_check(v, v8t, v_scale, dtype, B, N, S, D, v_sb, v_sn, v_ss);
+  if (rc != MSD_OK) return rc;
+  if (!workspace) return MSD_ERR_BAD_ARG;
+  if (ws_bytes < mindiesd_fp8_v_quant_workspace_size(B, N)) return MSD_ERR_WORKSPACE;
+  return v_quant_launch(v, v8t, v_scale, dtype, B, N, S, v_sb, v_sn, v_ss, (unsigned*)workspace, stream);
+}
+
+// ---- the same without any allocation on the caller's or the library's side ------------------------------------
+// The per-channel maxima live in a device array that is part of the library's code object: every GPU the library
+// runs on holds its own copy (2 MiB) at its own address until the process ends.  `g_v_quant_scratch` names the
+// array for the device compiler only; host code must use the address hipGetSymbolAddress returns for the current
+// device, looked up once per device and kept in g_v_quant_scratch_ptr.
+static __device__ __align__(256) unsigned g_v_quant_scratch[MINDIESD_FP8_V_QUANT_STATIC_MAX_HEADS * 128];
+static unsigned* g_v_quant_scratch_ptr[kMaxDevices];
+static std::mutex g_v_quant_scratch_mutex;
+
+int mindiesd_fp8_v_quant_static_max_heads(void) { return MINDIESD_FP8_V_QUANT_STATIC_MAX_HEADS; }
+
+int mindiesd_fp8_v_quant_static(const void* v, void* v8t, float* v_scale, int dtype, int B, int N, int S, int D,
+                                long long v_sb, long long v_sn, long long v_ss, hipStream_t stream) {
+  const int rc = v_quant_check(v, v8t, v_scale, dtype, B, N, S, D, v_sb, v_sn, v_ss);
+  if (rc != MSD_OK) return rc;
+  if ((long long)B * N > MINDIESD_FP8_V_QUANT_STATIC_MAX_HEADS) return MSD_ERR_WORKSPACE;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MSD_ERR_LAUNCH;
+  unsigned* scratch;
+  {
+    std::lock_guard<std::mutex> guard(g_v_quant_scratch_mutex);
+    if (!g_v_quant_scratch_ptr[dev]) {
+      void* ptr = nullptr;
+      if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_v_quant_scratch)) != hipSuccess || !ptr) return MSD_ERR_LAUNCH;
+      g_v_quant_scratch_ptr[dev] = (unsigned*)ptr;
+    }
+    scratch = g_v_quant_scratch_ptr[dev];
+  }
+  return v_quant_launch(v, v8t, v_scale, dtype, B, N, S, v_sb, v_sn, v_ss, scratch, stream);
 }
 
 int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,

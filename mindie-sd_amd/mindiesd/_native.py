@@ -41,6 +41,8 @@ SIGNATURES = {
     "mindiesd_fa_rot_block_quant": (c_int, [c_p, c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_f, c_int, c_p]),
     "mindiesd_fp8_v_quant_workspace_size": (c_sz, [c_int, c_int]),
     "mindiesd_fp8_v_quant": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_p, c_sz, c_p]),
+    "mindiesd_fp8_v_quant_static_max_heads": (c_int, []),
+    "mindiesd_fp8_v_quant_static": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_p]),
     "mindiesd_fp8_attention_fwd": (c_int, [c_p] * 7 + [c_int] * 6 + [c_ll] * 3 + [c_f, c_int, c_p]),
     "mindiesd_mx_quant": (c_int, [c_p, c_p, c_p, c_int, c_ll, c_int, c_ll, c_p]),
     "mindiesd_mxfp8_gemm": (c_int, [c_p] * 6 + [c_int] * 5 + [c_p]),
