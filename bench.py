@@ -15,7 +15,6 @@ reference's unfused torch path) on a bounded sample of the same workload on the 
 """
 import argparse
 import json
-import math
 import os
 import sys
 import time
@@ -44,50 +43,7 @@ def attn_flops(cfg):
     return 4.0 * cfg["B"] * cfg["N"] * cfg["S"] * cfg["S"] * cfg["D"]
 
 
-# ---- synthetic inputs (seeded; generated on the device they are used on) ---------------------------
-def dense_inputs(cfg, device, seed=0, mul=0.5, dtype=None):
-    """q, k, v = mul * N(0,1), BNSD."""
-    import torch
-    dtype = dtype or torch.bfloat16
-    g = torch.Generator(device=device).manual_seed(seed)
-    shape = (cfg["B"], cfg["N"], cfg["S"], cfg["D"])
-    return tuple((torch.randn(shape, generator=g, device=device, dtype=torch.float32) * mul).to(dtype)
-                 for _ in range(3))
-
-
-def _gauss_kernel(sigma, device):
-    import torch
-    r = int(math.ceil(3 * sigma))
-    x = torch.arange(-r, r + 1, device=device, dtype=torch.float32)
-    k = torch.exp(-0.5 * (x / sigma) ** 2)
-    return k / k.sum()
-
-
-def smooth_field_inputs(cfg, device, seed=0, sigma=2.0, noise=0.3, heads=None, dtype=None):
-    """q, k, v (BNSD, tokens flattened T-H-W): per (head, channel) an N(0,1) field on the latent grid,
-    Gaussian filtered with sigma tokens along T, H and W (separable, zero padded), renormalised to
-    unit variance per head, plus ``noise`` * N(0,1).  Block scores are therefore structured."""
-    import torch
-    import torch.nn.functional as F
-    dtype = dtype or torch.bfloat16
-    t, h, w = cfg["grid"]
-    n, d = (cfg["N"] if heads is None else heads), cfg["D"]
-    g = torch.Generator(device=device).manual_seed(seed)
-    kern = _gauss_kernel(sigma, device)
-    r = kern.numel() // 2
-    outs = []
-    for _ in range(3):
-        heads_out = []
-        for _n in range(n):
-            f = torch.randn((d, 1, t, h, w), generator=g, device=device)
-            f = F.conv3d(f, kern.view(1, 1, -1, 1, 1), padding=(r, 0, 0))
-            f = F.conv3d(f, kern.view(1, 1, 1, -1, 1), padding=(0, r, 0))
-            f = F.conv3d(f, kern.view(1, 1, 1, 1, -1), padding=(0, 0, r))
-            f = f / f.std()
-            f = f + noise * torch.randn(f.shape, generator=g, device=device)
-            heads_out.append(f.reshape(d, t * h * w).t().to(dtype))
-        outs.append(torch.stack(heads_out, 0).unsqueeze(0).contiguous())
-    return tuple(outs)
+from workloads import dense_inputs, outlier_inputs, smooth_field_inputs  # noqa: E402  (seeded synthetic inputs)
 
 
 # ---- timing -----------------------------------------------------------------------------------------
@@ -228,18 +184,28 @@ def extra_sparse(device, steps, warmup, dense_ms):
     }
 
 
-def outlier_inputs(cfg, device, seed=0, dtype=None):
-    """q, k, v = N(0,1) with 1 % of the elements (seeded Bernoulli) scaled by 8, BNSD."""
+def extra_ada_bsa(device, steps, warmup, dense_ms):
+    """Adaptive block-sparse attention (ada_bsa) at the 14B 720p shape on the smooth-field inputs: mask estimate
+    (strided scores + block selection) and attention over the estimated mask."""
     import torch
-    dtype = dtype or torch.bfloat16
-    g = torch.Generator(device=device).manual_seed(seed)
-    shape = (cfg["B"], cfg["N"], cfg["S"], cfg["D"])
-    outs = []
-    for _ in range(3):
-        x = torch.randn(shape, generator=g, device=device)
-        m = torch.rand(shape, generator=g, device=device) < 0.01
-        outs.append(torch.where(m, x * 8, x).to(dtype))
-    return tuple(outs)
+    from mindiesd.layers.flash_attn import ada_bsa
+    cfg = CFG_14B_720P
+    q, k, v = smooth_field_inputs(cfg, device, seed=3)
+    scale = cfg["D"] ** -0.5
+    est = lambda: ada_bsa.sparse_block_estimate(q, k, scale_value=scale / 8, threshold=0.9, row_sparse=0.25)
+    smask, sct = est()
+    nb = (cfg["S"] + 127) // 128
+    density = float(smask[..., :nb].float().mean())
+    est_ms, _ = time_steps(est, steps, warmup)
+    att = lambda: ada_bsa.ada_block_sparse_attention(q, k, v, smask, sct, scale_value=scale)
+    att_ms, _ = time_steps(att, steps, warmup)
+    em, am = median(est_ms), median(att_ms)
+    est_flops = 2.0 * cfg["N"] * (cfg["S"] / 8) ** 2 * 8 * cfg["D"]
+    return {"workload": "ada_bsa B1 N40 S75600 D128, cdf threshold 0.9, at most 25 % of the key blocks per row, "
+                        "smooth-field inputs",
+            "mask_density": density, "estimate_ms": em, "estimate_tflops": est_flops / em / 1e9,
+            "attention_ms": am, "total_ms": em + am, "speedup_vs_dense": dense_ms / (em + am),
+            "attention_speedup_vs_dense": dense_ms / am}
 
 
 def extra_fp8(device, steps, warmup):
@@ -341,7 +307,7 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference kernel for scaling rocprof byte counters)")
     ap.add_argument("--extras-only", default="",
-                    help="comma separated subset of extras to run (dense_wan1p3b,causal_varlen,sparse_rf_v3,fp8_attention,"
+                    help="comma separated subset of extras to run (dense_wan1p3b,causal_varlen,sparse_rf_v3,ada_bsa,fp8_attention,"
                          "mxfp8_gemm_swiglu)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -396,6 +362,7 @@ def main():
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
                          ("causal_varlen", lambda: extra_causal_varlen(device, args.steps, args.warmup)),
                          ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
+                         ("ada_bsa", lambda: extra_ada_bsa(device, args.steps, args.warmup, kernel_ms)),
                          ("fp8_attention", lambda: extra_fp8(device, args.steps, args.warmup)),
                          ("mxfp8_gemm_swiglu", lambda: extra_gemm(device, args.steps, args.warmup))):
             if args.extras_only and name not in args.extras_only.split(","):

@@ -125,23 +125,28 @@ int mindiesd_ada_block_sparse_attention_fwd(const void* q, const void* k, const 
                                             float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
                                             int causal, hipStream_t stream);
 
-/* Mask estimate, steps 2 and 3 of aclnnSparseBlockEstimate (csrc/plugin/sparse_block_estimate.cpp:27-85,
+/* Mask estimate: aclnnSparseBlockEstimate (csrc/plugin/sparse_block_estimate.cpp:27-85,
  * csrc/ops/sparse_block_estimate/op_kernel/sparse_block_estimate.h; numpy statement
- * tests/plugin/test_sparseblockestimate.py:49-145).  Step 1, the strided anti-diagonal score matrix
- * P'[i][j] = sum_{s<8} q[8i+7-s] . k[8j+s], is a plain [Sr, 8D] x [8D, Sr] GEMM (Sr = ceil(S/8)) that the
- * caller computes with a GEMM library and passes as pmat [BN][Sr][ldp] (16-bit, ldp % 8 == 0).
- * mindiesd_sbe_block_scores: scores[bn][I][J] = sum over the 16 x 16 block (I, J) of softmax_j(scale * P'),
- *   fp32 [BN][NB][NB], NB = ceil(Sr / 16).
- * mindiesd_sbe_select: per row, key blocks in descending score order (the last block left out) are kept
- *   until their running sum reaches threshold * total, at most row_sparse * NB of them; the first block is
- *   kept if keep_sink, the last if keep_recent.  mask int8 [BN][NB][pitch] (pitch >= NB, zero padded; the
- *   reference uses pitch = NB rounded up to 32), count int32 [BN][NB].
- * causal != 0 (test_sparseblockestimate.py:71-78, 121-127): the block rows of one step of 1024 query tokens see
- *   the strided columns below min(col_cap, 128 * (step + 1)) with col_cap = S / 8; row i of the selection ranks
- *   its first i + 1 blocks with the diagonal block in the place of the last one, rows 0 and 1 keep their whole
- *   prefix, blocks above the diagonal are never selected. */
-int mindiesd_sbe_block_scores(const void* pmat, float* scores, int dtype, int BN, int Sr, int ldp, float scale,
-                              int causal, int col_cap, hipStream_t stream);
+ * tests/plugin/test_sparseblockestimate.py:49-145) in two calls.
+ * mindiesd_sbe_scores: q [B][N][S][128], k [B][Nkv][S][128] (element strides as above) -> scores fp32
+ *   [B * N][NB][NB], NB = ceil(S / 128): scores[bn][I][J] = sum over the 16 x 16 block (I, J) of
+ *   softmax_j(scale * P'), with the anti-diagonal strided products P'[i][j] = sum_{s<8} q[8i+7-s] . k[8j+s]
+ *   (tokens past S count as zeros; the caller passes scale = softmax scale / 8).  P' is never stored.
+ *   workspace: mindiesd_sbe_scores_workspace_size(B * N, S) bytes, or less - any size that holds one head works,
+ *   the heads are then processed in groups.
+ *   causal != 0 (test_sparseblockestimate.py:71-78): the rows of one step of 1024 query tokens see the strided
+ *   columns below min(S / 8, 128 * (step + 1)); scores beyond are zero.
+ * mindiesd_sbe_select (sparse_block_estimate.h:947-1078): per block row, the key blocks take part that the row may
+ *   see (all NB, or with causal the first I + 1; causal rows with at most 2 keep them all).  The last of them (if
+ *   keep_recent or not causal) and the first (if keep_sink) are left out of the ranking and forced afterwards; the
+ *   others are kept in descending score order until their running sum reaches threshold * their total
+ *   (threshold >= 1 keeps all), at most row_sparse * blocks of them when at least 10 take part; block 0 is always
+ *   kept.  mask int8 [BN][NB][pitch] (pitch >= NB, zero padded; the reference uses NB rounded up to 32), count
+ *   int32 [BN][NB]. */
+size_t mindiesd_sbe_scores_workspace_size(int heads, int S);
+int mindiesd_sbe_scores(const void* q, const void* k, float* scores, int dtype, int B, int N, int Nkv, int S, int D,
+                        long long q_sb, long long q_sn, long long q_ss, long long k_sb, long long k_sn, long long k_ss,
+                        float scale, int causal, void* workspace, size_t ws_bytes, hipStream_t stream);
 int mindiesd_sbe_select(const float* scores, signed char* mask, int* count, int BN, int NB, int pitch,
                         float threshold, float row_sparse, int keep_sink, int keep_recent, int causal,
                         hipStream_t stream);

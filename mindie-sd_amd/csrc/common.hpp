@@ -133,6 +133,14 @@ __device__ __forceinline__ float half_sum(float v) {
   return lo + hi;
 }
 
+// Sums over the two wave halves of two values at once: lanes 0..31 receive the total of x, lanes 32..63 the total
+// of y (the swap leaves x's lower and y's lower half in one register, their upper halves in the other).
+__device__ __forceinline__ float half_pair_sum(float x, float y) {
+  float a = x, b = y;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+
 // The same across the four 16-lane rows of a wavefront: v_permlane16_swap exchanges the odd rows of its first
 // operand with the even rows of its second, so with both holding v one result has rows (0, 0, 2, 2) of v and
 // the other rows (1, 1, 3, 3); combining them and then the two halves leaves the result of all four rows in

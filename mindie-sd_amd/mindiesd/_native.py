@@ -26,7 +26,8 @@ SIGNATURES = {
     "mindiesd_flash_attention_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p]),
     "mindiesd_flash_attention_general_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_int, c_p] + [c_ll] * 3 + [c_p]),
     "mindiesd_ada_block_sparse_attention_fwd": (c_int, [c_p] * 4 + [c_int] * 6 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_int, c_p]),
-    "mindiesd_sbe_block_scores": (c_int, [c_p, c_p] + [c_int] * 4 + [c_f, c_int, c_int, c_p]),
+    "mindiesd_sbe_scores_workspace_size": (c_sz, [c_int, c_int]),
+    "mindiesd_sbe_scores": (c_int, [c_p, c_p, c_p] + [c_int] * 6 + [c_ll] * 6 + [c_f, c_int, c_p, c_sz, c_p]),
     "mindiesd_sbe_select": (c_int, [c_p, c_p, c_p] + [c_int] * 3 + [c_f, c_f, c_int, c_int, c_int, c_p]),
     "mindiesd_set_dense_variant": (None, [c_int]),
     "mindiesd_block_sparse_attention_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_p, c_p]),

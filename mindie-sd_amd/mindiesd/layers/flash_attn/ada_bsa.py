@@ -3,9 +3,9 @@ attention over the estimated mask (ada_block_sparse_attention).
 
 Stands where the reference's torch ops call its in-tree AscendC kernels
 (csrc/plugin/sparse_block_estimate.cpp:27-85, csrc/plugin/ada_block_sparse_attention.cpp:27-57).
-The estimate is three steps: the anti-diagonal strided score matrix P' (a plain GEMM, handed to the GEMM
-library through torch.bmm), its row softmax summed over 16 x 16 blocks, and the per-row selection of key
-blocks; the last two are HIP kernels of this library.
+The estimate is two launches of this library: the block scores (anti-diagonal strided products, their row
+softmax and the sums over 16 x 16 blocks in one kernel that reads q and k in place) and the per-row selection
+of key blocks.
 """
 import torch
 
@@ -15,20 +15,9 @@ from .hip_flash_attn import HEAD_DIM, _strides_bns
 from .rainfusion import BLOCK, _aligned, _check_gpu16, _dims, mask_to_lists
 
 STRIDE = 8
-# Heads are processed in groups whose P' matrices together stay below 2^30 elements (2 GiB in 16 bits).
-_PMAT_ELEMS = 1 << 30
-# Longest sequence the estimate accepts.  Runs at 32760 and 75600 tokens ended in a GPU memory fault whose
-# cause has not been established (the kernels' index arithmetic checks out on paper; sequences up to 3000
-# tokens pass their parity tests), so longer sequences are refused until it is.
-MAX_ESTIMATE_TOKENS = 3072
-
-
-def _to_bnsd(t, layout):
-    if layout == "BNSD":
-        return t
-    if layout == "BSND":
-        return t.transpose(1, 2)
-    raise RuntimeError(f"input_layout only supports 'BNSD' and 'BSND', got {layout}")
+# Scratch of the score kernel is allocated up to this size; with more heads than fit, the library goes
+# through them in groups.
+_WORKSPACE_BYTES = 1 << 30
 
 
 def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size=128, scale_value=1.0, threshold=1.0,
@@ -37,51 +26,34 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
     ``scale_value`` multiplies the strided products (the caller passes softmax_scale / stride)."""
     for name, t in (("query", query), ("key", key)):
         _check_gpu16(t, name)
-    if query.dim() != 4 or key.dim() != 4:
-        raise RuntimeError("sparse_block_estimate expects 4-D query and key")
+    if input_layout not in ("BNSD", "BSND"):
+        raise RuntimeError(f"input_layout only supports 'BNSD' and 'BSND', got {input_layout}")
     if stride != STRIDE or sparse_size != BLOCK:
         raise RuntimeError(f"sparse_block_estimate supports stride {STRIDE} and sparse_size {BLOCK} only, "
                            f"got {stride} and {sparse_size}")
-    s_tokens = query.shape[2] if input_layout == "BNSD" else query.shape[1]
-    if s_tokens > MAX_ESTIMATE_TOKENS:
-        raise RuntimeError(f"sparse_block_estimate: sequences longer than {MAX_ESTIMATE_TOKENS} tokens are switched off in "
-                           f"this build (got {s_tokens})")
-    q, k = _to_bnsd(query, input_layout), _to_bnsd(key, input_layout)
-    b, n, s, d = q.shape
-    if k.shape[0] != b or k.shape[2] != s or k.shape[3] != d or n % k.shape[1] != 0 or k.dtype != q.dtype:
+    q, k = _aligned(query), _aligned(key)
+    b, n, s = _dims(q, input_layout)
+    kb, nkv, ks = _dims(k, input_layout)
+    if kb != b or ks != s or nkv == 0 or n % nkv != 0 or k.dtype != q.dtype:
         raise RuntimeError("sparse_block_estimate: query and key must have the same batch, length, head_dim and dtype")
-    if k.shape[1] != n:
-        k = k.repeat_interleave(n // k.shape[1], dim=1)
-    sp = (s + STRIDE - 1) // STRIDE * STRIDE
-    sr = sp // STRIDE
-    ldp = (sr + 7) // 8 * 8
     nb = (s + BLOCK - 1) // BLOCK
     pitch = (nb + 31) // 32 * 32
-    # Q': the 8 tokens of a group in reverse order, side by side; K': in order; tokens past S are zeros
-    qp = torch.zeros((b, n, sp, d), dtype=q.dtype, device=q.device)
-    qp[:, :, :s] = q
-    qp = qp.view(b * n, sr, STRIDE, d).flip(2).reshape(b * n, sr, STRIDE * d)
-    kp = torch.zeros((b * n, ldp, STRIDE * d), dtype=q.dtype, device=q.device)
-    kp[:, :sr].view(b * n, sr * STRIDE, d)[:, :s] = k.reshape(b * n, s, d)
-    scores = torch.empty((b * n, nb, nb), dtype=torch.float32, device=q.device)
-    if sr * ldp > _PMAT_ELEMS:
-        raise RuntimeError(f"sparse_block_estimate: sequence length {s} is beyond what this build estimates")
-    group = max(1, min(b * n, _PMAT_ELEMS // (sr * ldp)))
     lib = _native.lib()
+    scores = torch.empty((b * n, nb, nb), dtype=torch.float32, device=q.device)
+    one_head = lib.mindiesd_sbe_scores_workspace_size(1, s)
+    ws_bytes = min(one_head * b * n, max(one_head, _WORKSPACE_BYTES // one_head * one_head))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    mask = torch.empty((b, n, nb, pitch), dtype=torch.int8, device=q.device)
+    count = torch.empty((b, n, nb), dtype=torch.int32, device=q.device)
     with torch.cuda.device(q.device):
-        for g0 in range(0, b * n, group):
-            g1 = min(b * n, g0 + group)
-            pmat = torch.bmm(qp[g0:g1], kp[g0:g1].transpose(1, 2))  # [g, sr, ldp] raw strided products
-            rc = lib.mindiesd_sbe_block_scores(pmat.data_ptr(), scores[g0:g1].data_ptr(), _native.DTYPE_CODE[q.dtype],
-                                               g1 - g0, sr, ldp, float(scale_value), int(bool(causal)),
-                                               max(1, s // STRIDE), _native.stream_ptr(q.device))
-            _native.check(rc, "mindiesd_sbe_block_scores")
-            del pmat
-        mask = torch.empty((b, n, nb, pitch), dtype=torch.int8, device=q.device)
-        count = torch.empty((b, n, nb), dtype=torch.int32, device=q.device)
+        stream = _native.stream_ptr(q.device)
+        rc = lib.mindiesd_sbe_scores(q.data_ptr(), k.data_ptr(), scores.data_ptr(), _native.DTYPE_CODE[q.dtype], b, n,
+                                     nkv, s, HEAD_DIM, *_strides_bns(q, input_layout), *_strides_bns(k, input_layout),
+                                     float(scale_value), int(bool(causal)), ws.data_ptr(), ws_bytes, stream)
+        _native.check(rc, "mindiesd_sbe_scores")
         rc = lib.mindiesd_sbe_select(scores.data_ptr(), mask.data_ptr(), count.data_ptr(), b * n, nb, pitch,
                                      float(threshold), float(row_sparse), int(bool(keep_sink)), int(bool(keep_recent)),
-                                     int(bool(causal)), _native.stream_ptr(q.device))
+                                     int(bool(causal)), stream)
         _native.check(rc, "mindiesd_sbe_select")
     if return_scores:
         return mask, count, scores.view(b, n, nb, nb)

@@ -28,7 +28,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_mas
     (index-list and int8-mask variants; both need ``latent_shape_q`` = (t, h, w) with
     t*h*w + txt_len == S, ``block_size`` 128 and ``sparsity`` in [0, 1)); 'ada_bsa' = adaptive block
     sparsity (mask estimated from strided anti-diagonal scores, ``cdf_threshold``, ``sparsity`` as the cap,
-    ``keep_sink`` / ``keep_recent``; non-causal estimation only).
+    ``keep_sink`` / ``keep_recent``, ``is_causal``).
     The output has the layout, dtype and token order of ``q``."""
     check_params(input_layout, sparse_type)
     head_dim = q.shape[-1]

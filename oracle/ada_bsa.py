@@ -6,7 +6,10 @@ Restates the numpy statements the reference's tests hold for its two in-tree Asc
 tests/plugin/test_adablocksparseattention.py:35-87.  The reference's test exercises the non-causal estimate only
 (test_sparseblockestimate.py:166); the causal branches of its numpy statement are restated as they stand.  Its
 own tolerance for the estimate is a mask difference below 2 % of the selected blocks and fewer than 1 % omitted
-blocks (:231-241).
+blocks (:231-241).  The selection exists twice in the reference: as that numpy statement (``select_blocks``) and as
+the kernel's ScoreCompute (csrc/ops/sparse_block_estimate/op_kernel/sparse_block_estimate.h:947-1078, restated as
+``select_blocks_kernel``); they differ in how the first block and the switches are treated, and the product
+follows the kernel.
 """
 import numpy as np
 import torch
@@ -94,9 +97,49 @@ def select_blocks(score_row, threshold, force_sparse, keep_sink=True, keep_recen
     return to_sort >= guard
 
 
+SBE_EPS = 1e-5  # sparse_block_estimate.h:85
+
+
+def select_blocks_kernel(score_row, threshold, row_sparse, keep_sink=True, keep_recent=True, causal=False):
+    """The reference kernel's selection for one row (ScoreCompute, sparse_block_estimate.h:947-1078);
+    ``score_row`` holds the columns that take part (all blocks, or with ``causal`` those up to the diagonal).
+    Differences from ``select_blocks``: the first block is left out of the ranking and of the total when
+    ``keep_sink`` (setFirst) is set and is kept in any case (:1067); without ``causal`` the last block is left
+    out and forced whatever ``keep_recent`` (setDiag) says (:976-978, :1051-1053); the cap only applies from 10
+    columns on (:1046); a threshold >= 1 keeps every column (:1042-1045); the guard is lowered by 1e-5 (:1047)."""
+    src = np.array(score_row, dtype=np.float32).copy()
+    n = src.shape[0]
+    if causal and n <= 2:                                    # :958-962
+        return np.ones(n, dtype=np.bool_)
+    last_out = keep_recent or not causal
+    if last_out:                                             # :976-978: the mask of ranked columns stops before it
+        src[-1] = 0
+    if keep_sink:                                            # :980-983
+        src[0] = 0
+    ranked = -np.sort(-src, kind="stable")                   # :996
+    if threshold < 1.0:                                      # :1009-1041: first column at which the running sum
+        run = np.cumsum(ranked, dtype=np.float32)            # reaches threshold * total (:991 total of the ranked ones)
+        hit = np.nonzero(run >= np.float32(threshold) * run[-1])[0]
+        cnt = int(hit[0]) if hit.size else n - 1
+        guard = np.float32(ranked[cnt])
+    else:                                                    # :1042-1045
+        cnt, guard = n, np.float32(0.0)
+    if cnt > n * row_sparse and n >= 10:                     # :1046-1049
+        guard = np.float32(ranked[max(int(n * row_sparse), 1) - 1])
+    guard = np.float32(guard - np.float32(SBE_EPS))          # :1047
+    if keep_sink:                                            # :1048-1050
+        src[0] = guard + 1
+    if last_out:                                             # :1051-1053
+        src[-1] = guard + 1
+    keep = src > guard                                       # :1056-1066: relu(x - guard) / (relu + 0.001), rounded up
+    keep[0] = True                                           # :1067
+    return keep
+
+
 def sparse_estimate(query, key, blocksize=128, stride=8, threshold=0.5, force_sparse=1.0, keep_sink=True,
-                    keep_recent=True, causal=False):
+                    keep_recent=True, causal=False, rules="numpy"):
     """[B, N, S, D] query / key (any float dtype) -> boolean mask [B, N, nb, nb], nb = ceil(S / blocksize).
+    ``rules``: 'numpy' = the selection of the reference's numpy statement, 'kernel' = that of its kernel.
     ``causal`` (:121-127, :140): row i selects among its first i + 1 blocks, the diagonal block standing where
     the last block stands otherwise (forced only with ``keep_recent``, the kernel's setDiag,
     sparse_block_estimate.h:1047-1049); rows 0 and 1 keep their whole prefix."""
@@ -109,13 +152,14 @@ def sparse_estimate(query, key, blocksize=128, stride=8, threshold=0.5, force_sp
         for ni in range(nq):
             sc = block_scores(qf[bi, ni], kf[bi, ni // gqa], blocksize, stride, causal)
             for i in range(nb):
-                if not causal:
-                    mask[bi, ni, i] = select_blocks(sc[i, :nb], threshold, force_sparse, keep_sink, keep_recent)
-                elif i <= 1:
-                    mask[bi, ni, i, :i + 1] = True
+                n = i + 1 if causal else nb
+                if rules == "kernel":
+                    mask[bi, ni, i, :n] = select_blocks_kernel(sc[i, :n], threshold, force_sparse, keep_sink,
+                                                               keep_recent, causal)
+                elif causal and i <= 1:
+                    mask[bi, ni, i, :n] = True
                 else:
-                    mask[bi, ni, i, :i + 1] = select_blocks(sc[i, :i + 1], threshold, force_sparse, keep_sink,
-                                                            keep_recent)
+                    mask[bi, ni, i, :n] = select_blocks(sc[i, :n], threshold, force_sparse, keep_sink, keep_recent)
     return mask
 
 

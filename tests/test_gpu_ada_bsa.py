@@ -24,6 +24,13 @@ def _structured(shape, seed, dtype):
     return (base + 0.5 * _rand(shape, seed + 1, torch.float32)).to(dtype)
 
 
+def _mask_close(got, want):
+    """The reference's tolerance for its kernel against its numpy statement (test_sparseblockestimate.py:231-241)."""
+    selected = want.sum()
+    assert (got != want).sum() / selected < 0.02, ((got != want).sum(), selected)
+    assert (got < want).sum() / selected < 0.01, ((got < want).sum(), selected)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("s,threshold,row_sparse", [(2048, 0.85, 1.0), (3000, 0.6, 0.5), (1031, 0.9, 1.0)])
 def test_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, dtype):
@@ -39,13 +46,57 @@ def test_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, dtype):
     got = smask.cpu().numpy().astype(bool)
     assert not got[..., nb:].any()
     assert np.array_equal(sct.cpu().numpy(), got.sum(-1))
-    want = oab.sparse_estimate(q, k, threshold=threshold, force_sparse=row_sparse)
+    want = oab.sparse_estimate(q, k, threshold=threshold, force_sparse=row_sparse, rules="kernel")
     got = got[..., :nb]
     assert got[..., 0].all() and got[..., -1].all()
     for h in range(2):
-        selected = want[0, h].sum()
-        assert (got[0, h] != want[0, h]).sum() / selected < 0.02
-        assert (got[0, h] < want[0, h]).sum() / selected < 0.01
+        _mask_close(got[0, h], want[0, h])
+
+
+def test_estimate_against_the_numpy_statement_on_the_reference_test_case(cuda):
+    """The reference's own test (tests/plugin/test_sparseblockestimate.py:150-241): B1 N1 S8192 D128, N(0,1) inputs
+    cast to fp16, threshold 0.85, no cap, default switches, kernel against the numpy statement within 2 % / 1 %."""
+    import mindiesd  # noqa: F401
+    q, k = _rand((1, 1, 8192, 128), 0), _rand((1, 1, 8192, 128), 1)
+    smask, sct = torch.ops.mindiesd.sparse_block_estimate(
+        q.to(cuda), k.to(cuda), input_layout="BNSD", stride=8, sparse_size=128, num_heads=1, num_key_value_heads=1,
+        scale_value=128 ** -0.5 / 8, threshold=0.85, causal=False, keep_sink=True, keep_recent=True, row_sparse=1.0)
+    assert smask.shape == (1, 1, 64, 64) and sct.shape == (1, 1, 64)
+    want = oab.sparse_estimate(q, k, threshold=0.85, force_sparse=1.0, rules="numpy")
+    _mask_close(smask.cpu().numpy().astype(bool)[0, 0], want[0, 0])
+
+
+@pytest.mark.parametrize("layout", ["BNSD", "BSND"])
+def test_block_scores_layouts_heads_and_workspace_groups(cuda, layout):
+    """Scores of the fused kernel against the oracle's block scores: grouped-query heads, both layouts, a batch,
+    a sequence that is no multiple of 8, and a workspace that only holds two of the six heads at a time."""
+    from mindiesd import _native
+    s, b, n, nkv = 2707, 2, 3, 1
+    q, k = _structured((b, n, s, 128), 31, torch.bfloat16), _structured((b, nkv, s, 128), 33, torch.bfloat16)
+    qd, kd = (t.to(cuda) if layout == "BNSD" else t.transpose(1, 2).contiguous().to(cuda).transpose(1, 2) for t in (q, k))
+    nb = (s + 127) // 128
+    lib = _native.lib()
+    scores = torch.full((b * n, nb, nb), -1.0, dtype=torch.float32, device=cuda)
+    ws_bytes = lib.mindiesd_sbe_scores_workspace_size(2, s)
+    assert ws_bytes * 3 == lib.mindiesd_sbe_scores_workspace_size(6, s)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    rc = lib.mindiesd_sbe_scores(qd.data_ptr(), kd.data_ptr(), scores.data_ptr(), 0, b, n, nkv, s, 128,
+                                 qd.stride(0), qd.stride(1), qd.stride(2), kd.stride(0), kd.stride(1), kd.stride(2),
+                                 128 ** -0.5 / 8, 0, ws.data_ptr(), ws_bytes, _native.stream_ptr(cuda))
+    assert rc == 0
+    got = scores.cpu().numpy().reshape(b, n, nb, nb)
+    for bi in range(b):
+        for ni in range(n):
+            want = oab.block_scores(q[bi, ni].float().numpy(), k[bi, 0].float().numpy())
+            assert np.abs(got[bi, ni] - want).max() < 2e-3, (bi, ni, np.abs(got[bi, ni] - want).max())
+            assert abs(got[bi, ni].sum() - (s + 7) // 8) < 0.05
+    # too small a workspace and bad arguments are refused
+    assert lib.mindiesd_sbe_scores(qd.data_ptr(), kd.data_ptr(), scores.data_ptr(), 0, b, n, nkv, s, 128,
+                                   qd.stride(0), qd.stride(1), qd.stride(2), kd.stride(0), kd.stride(1), kd.stride(2),
+                                   0.01, 0, ws.data_ptr(), ws_bytes // 2 - 16, _native.stream_ptr(cuda)) == 3
+    assert lib.mindiesd_sbe_scores(qd.data_ptr(), kd.data_ptr(), scores.data_ptr(), 0, b, n, nkv, s, 64,
+                                   qd.stride(0), qd.stride(1), qd.stride(2), kd.stride(0), kd.stride(1), kd.stride(2),
+                                   0.01, 0, ws.data_ptr(), ws_bytes, _native.stream_ptr(cuda)) == 2
 
 
 @pytest.mark.parametrize("keep_recent", [True, False])
@@ -66,36 +117,33 @@ def test_causal_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, 
     assert got[0, :, 0, 0].all() and got[0, :, 1, :2].all()
     want_sc = oab.block_scores(q[0, 0].float().numpy(), k[0, 0].float().numpy(), causal=True)
     got_sc = scores.cpu().numpy()[0, 0]
-    assert np.abs(np.tril(got_sc) - np.tril(want_sc[:nb, :nb])).max() < 2e-2
+    assert np.abs(got_sc[:, :want_sc.shape[1]] - want_sc[:nb, :nb]).max() < 2e-3
     want = oab.sparse_estimate(q, k, threshold=threshold, force_sparse=row_sparse, keep_recent=keep_recent,
-                               causal=True)
+                               causal=True, rules="kernel")
     for h in range(2):
-        selected = want[0, h].sum()
-        assert (got[0, h] != want[0, h]).sum() / selected < 0.02
-        assert (got[0, h] < want[0, h]).sum() / selected < 0.01
+        _mask_close(got[0, h], want[0, h])
     if keep_recent:
         assert np.diag(got[0, 0]).all()
 
 
-def test_block_scores_and_selection_separately(cuda):
+@pytest.mark.parametrize("keep_sink,keep_recent", [(True, True), (False, True), (True, False), (False, False)])
+def test_block_scores_and_selection_separately(cuda, keep_sink, keep_recent):
     from mindiesd.layers.flash_attn.ada_bsa import sparse_block_estimate
     s = 2500
     q, k = _structured((1, 1, s, 128), 5, torch.float16), _structured((1, 1, s, 128), 7, torch.float16)
     mask, cnt, scores = sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=128 ** -0.5 / 8, threshold=0.8,
-                                              row_sparse=0.7, return_scores=True)
+                                              row_sparse=0.7, keep_sink=keep_sink, keep_recent=keep_recent,
+                                              return_scores=True)
     want = oab.block_scores(q[0, 0].float().numpy(), k[0, 0].float().numpy())
     got = scores.cpu().numpy()[0, 0]
     nb = (s + 127) // 128
     assert got.shape == (nb, nb)
-    # 16-bit products in the logits: block masses agree to a fraction of a percent of a row's mass (16)
-    assert np.abs(got - want).max() < 2e-2 and abs(got.sum() - (s + 7) // 8) < 0.5
-    # the selection kernel on the GPU's own scores reproduces the statement row by row
-    sel = np.stack([oab.select_blocks(got[i], 0.8, 0.7) for i in range(nb)])
+    # exact 16-bit inputs, fp32 accumulation: block masses agree to a small fraction of a row's mass (16)
+    assert np.abs(got - want).max() < 2e-3 and abs(got.sum() - (s + 7) // 8) < 0.05
+    # the selection kernel on the GPU's own scores reproduces the kernel rules row by row
+    sel = np.stack([oab.select_blocks_kernel(got[i], 0.8, 0.7, keep_sink, keep_recent) for i in range(nb)])
     assert (mask.cpu().numpy()[0, 0, :, :nb].astype(bool) != sel).mean() < 1e-3
-    # switches: without the forced blocks fewer (or equal) blocks are kept
-    m2, c2 = sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=128 ** -0.5 / 8, threshold=0.8, row_sparse=0.7,
-                                   keep_sink=False, keep_recent=False)
-    assert bool((c2 <= cnt).all())
+    assert np.array_equal(cnt.cpu().numpy()[0, 0], mask.cpu().numpy()[0, 0].sum(-1))
 
 
 @pytest.mark.parametrize("layout", ["BNSD", "BSND"])
@@ -142,14 +190,30 @@ def test_sparse_attention_front_door_ada_bsa(cuda):
     assert 0.05 < density <= 0.75
 
 
-@pytest.mark.skip(reason="the estimate at 32760 tokens (B1 N12) and 75600 tokens (B1 N40) ended in a GPU memory fault "
-                         "whose cause is not established; sequences beyond 3072 tokens are refused by the host code")
-def test_sparse_block_estimate_long_sequences(cuda):
+@pytest.mark.parametrize("shape,check_heads", [((1, 12, 32760, 128), (0, 11)), ((1, 40, 75600, 128), (39,))])
+def test_sparse_block_estimate_long_sequences(cuda, shape, check_heads):
+    """The two DiT shapes (Wan2.1-1.3B and 14B 720p): block scores of the checked heads against the oracle, unit mass
+    per strided row in every head, masks of the checked heads within the reference's tolerance."""
     from mindiesd.layers.flash_attn import ada_bsa
-    q = _structured((1, 12, 32760, 128), 21, torch.bfloat16).to(cuda)
-    k = _structured((1, 12, 32760, 128), 23, torch.bfloat16).to(cuda)
-    mask, cnt = ada_bsa.sparse_block_estimate(q, k, scale_value=128 ** -0.5 / 8, threshold=0.9, row_sparse=0.25)
-    assert mask.shape == (1, 12, 256, 256) and int(cnt.min()) >= 2
+    b, n, s, d = shape
+    q = torch.cat([_structured((1, 1, s, d), 21 + 2 * h, torch.bfloat16) for h in range(n)], dim=1)
+    k = torch.cat([_structured((1, 1, s, d), 121 + 2 * h, torch.bfloat16) for h in range(n)], dim=1)
+    print(f"estimate at {shape}", flush=True)
+    mask, cnt, scores = ada_bsa.sparse_block_estimate(q.to(cuda), k.to(cuda), scale_value=d ** -0.5 / 8, threshold=0.9,
+                                                      row_sparse=0.25, return_scores=True)
+    nb = (s + 127) // 128
+    assert mask.shape == (1, n, nb, (nb + 31) // 32 * 32) and int(cnt.min()) >= 2
+    sc = scores.cpu().numpy()[0]
+    rows = np.full(nb, 16.0)
+    rows[-1] = (s + 7) // 8 - 16 * (nb - 1)
+    assert np.abs(sc.sum(-1) - rows).max() < 1e-2          # every strided row carries probability mass 1
+    got = mask.cpu().numpy().astype(bool)[0, :, :, :nb]
+    assert np.array_equal(cnt.cpu().numpy()[0], got.sum(-1))
+    for h in check_heads:
+        want_sc = oab.block_scores(q[0, h].float().numpy(), k[0, h].float().numpy())
+        assert np.abs(sc[h] - want_sc).max() < 2e-3, (h, np.abs(sc[h] - want_sc).max())
+        want = np.stack([oab.select_blocks_kernel(want_sc[i], 0.9, 0.25) for i in range(nb)])
+        _mask_close(got[h], want)
 
 
 def test_ada_bsa_errors(cuda):
@@ -159,9 +223,6 @@ def test_ada_bsa_errors(cuda):
         torch.ops.mindiesd.sparse_block_estimate(q, q, input_layout="TND", causal=False)
     with pytest.raises(RuntimeError):
         torch.ops.mindiesd.sparse_block_estimate(q, q, stride=4, causal=False)
-    big = torch.zeros(1, 1, 3073, 128, dtype=torch.float16, device=cuda)
-    with pytest.raises(RuntimeError, match="switched off"):
-        torch.ops.mindiesd.sparse_block_estimate(big, big, causal=False)
     m = torch.ones(1, 1, 2, 32, dtype=torch.int8, device=cuda)
     c = torch.full((1, 1, 2), 2, dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError):

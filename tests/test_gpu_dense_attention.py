@@ -138,3 +138,27 @@ def test_errors(cuda):
         mindiesd.attention_forward(q[..., :64], q[..., :64], q[..., :64])
     with pytest.raises(ParametersInvalid):
         mindiesd.attention_forward(q, q, q, opt_mode="manual", op_type="nope")
+
+
+@pytest.mark.parametrize("s", [128, 300, 1153])
+def test_tail_tile_reads_nothing_past_the_sequence(cuda, s):
+    """K and V are views into slabs whose rows past the sequence hold NaN: the last key tile must take those rows
+    as zeros (the kernels rely on the range check of their buffer descriptors for that), otherwise 0 * NaN from
+    the second product shows up in the output."""
+    import mindiesd
+    q, k, v = _qkv((1, 2, s, 128), seed=s + 7)
+    slabs = []
+    for t in (k, v):
+        slab = torch.full((1, 2, s + 256, 128), float("nan"), dtype=torch.bfloat16, device=cuda)
+        slab[:, :, :s] = t.to(cuda)
+        slabs.append(slab[:, :, :s])
+    ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=True)
+    out = mindiesd.attention_forward(q.to(cuda), slabs[0], slabs[1], head_first=True).cpu()
+    assert not out.isnan().any()
+    _check(out, ref)
+    keep = torch.ones(s, s, dtype=torch.bool)
+    keep[:, s // 2] = False
+    ref = attention_math(q, k, v, keep, 128 ** -0.5, head_first=True)
+    out = mindiesd.attention_forward(q.to(cuda), slabs[0], slabs[1], attn_mask=keep.to(cuda), head_first=True).cpu()
+    assert not out.isnan().any()
+    _check(out, ref)

@@ -59,6 +59,50 @@ def test_select_blocks_hand_worked_rows():
     assert oab.select_blocks([0.3, 0.3, 0.3, 0.1], 0.4, 1.0).tolist() == [True, True, True, True]
 
 
+def test_select_blocks_kernel_hand_worked_rows():
+    """The kernel's own selection rules (sparse_block_estimate.h:947-1078) on rows worked out by hand."""
+    row = [0.5, 0.2, 0.1, 0.15, 0.05]
+    # sink and last block left out: ranked 0.2 0.15 0.1 0 0, total 0.45, 0.6 * 0.45 = 0.27 reached by the second
+    # (0.15), which is the guard; the guard itself passes (it is lowered by 1e-5), 0.1 does not
+    assert oab.select_blocks_kernel(row, 0.6, 1.0).tolist() == [True, True, False, True, True]
+    # both switches off, not causal: the last block is still left out and forced, the first is ranked:
+    # 0.5 0.2 0.15 0.1 0, total 0.95, 0.57 reached by the second (0.2)
+    assert oab.select_blocks_kernel(row, 0.6, 1.0, False, False).tolist() == [True, True, False, False, True]
+    # threshold 1: every column, also those without mass
+    assert oab.select_blocks_kernel([0.5, 0.0, 0.0, 0.5], 1.0, 1.0).all()
+    # the first block is kept even when nothing forces or ranks it
+    assert oab.select_blocks_kernel([0.0, 0.6, 0.3, 0.1], 0.5, 1.0, keep_sink=False).tolist() == [True, True, False, True]
+    # the cap applies from 10 columns on: 12 columns, 0.99 asks for nearly all, 0.25 * 12 = 3 ranked ones stay
+    row12 = [0.0, 0.3, 0.25, 0.2, 0.1, 0.05, 0.04, 0.03, 0.02, 0.005, 0.005, 0.0]
+    assert oab.select_blocks_kernel(row12, 0.99, 0.25).tolist() == [True, True, True, True] + [False] * 7 + [True]
+    assert oab.select_blocks_kernel(row12[:9], 0.99, 0.25).sum() > 5            # 9 columns: no cap
+    # causal: rows of at most two columns keep them all; the diagonal is ranked unless keep_recent leaves it out
+    assert oab.select_blocks_kernel([0.1, 0.9], 0.1, 0.1, causal=True).all()
+    diag_heavy = [0.05, 0.1, 0.05, 0.8]
+    assert oab.select_blocks_kernel(diag_heavy, 0.5, 1.0, keep_recent=False, causal=True).tolist() == [True, False, False, True]
+    assert oab.select_blocks_kernel(diag_heavy, 0.5, 1.0, keep_recent=True, causal=True).tolist() == [True, True, False, True]
+
+
+def test_kernel_rules_equal_the_numpy_statement_when_the_sink_carries_no_mass():
+    """With a first block of score 0 (nothing to leave out of the total), no cap and the default switches the two
+    statements of the selection are the same rule; rows whose guard has a near tie below it are left out, because
+    the kernel's lowered guard lets such a tie pass."""
+    rng = np.random.RandomState(0)
+    compared = 0
+    for _ in range(200):
+        n = int(rng.randint(3, 40))
+        row = rng.rand(n).astype(np.float32) ** 3
+        row[0] = 0
+        thr = float(rng.uniform(0.2, 0.95))
+        a, b = oab.select_blocks(row, thr, 1.0), oab.select_blocks_kernel(row, thr, 1.0)
+        if (a != b).any():
+            ranked = np.sort(row[:-1])
+            assert np.diff(ranked).min() < 2e-5, (row, thr)
+            continue
+        compared += 1
+    assert compared > 190
+
+
 def test_sparse_estimate_invariants():
     g = torch.Generator().manual_seed(0)
     q = torch.randn(1, 2, 1100, 32, generator=g)
@@ -127,3 +171,13 @@ def test_causal_scores_of_a_single_step_equal_the_plain_ones():
     a = oab.block_scores(q[0, 0].numpy(), k[0, 0].numpy(), causal=True)
     b = oab.block_scores(q[0, 0].numpy(), k[0, 0].numpy(), causal=False)
     assert np.array_equal(a, b)
+
+
+def test_causal_estimate_kernel_rules_invariants():
+    q, k = _qk(2100, 5)
+    m = oab.sparse_estimate(q, k, threshold=0.6, force_sparse=0.5, causal=True, rules="kernel")[0, 0]
+    assert not np.triu(m, 1).any() and m[:, 0].all() and np.diag(m).all()
+    full = oab.sparse_estimate(q, k, threshold=1.0, force_sparse=1.0, causal=True, rules="kernel")[0, 0]
+    assert np.array_equal(full, np.tril(np.ones_like(full)))
+    n = oab.sparse_estimate(q, k, threshold=0.7, force_sparse=1.0, rules="kernel")[0, 0]
+    assert n[:, 0].all() and n[:, -1].all()
