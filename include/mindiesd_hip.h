@@ -106,6 +106,26 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
                                                float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
                                                const int* token_order, hipStream_t stream);
 
+/* Block-sparse attention driven by the int8 mask itself (mask [B][N][ceil(Sq/128)][ceil(Skv/128)], non-zero =
+ * attend), in two passes over PAIRED query blocks: query blocks of a head whose mask rows overlap most are paired
+ * on the device; pass 1 computes, per pair, the key blocks both partners selected with one 256-row workgroup (each
+ * K/V tile is fetched once for both, the dense kernel's inner loop); pass 2 adds, per query block, the key blocks
+ * only it selected, continuing the running softmax of pass 1.  Same semantics as
+ * mindiesd_block_sparse_attention_fwd on the lists of the mask (results differ by the order of the accumulation
+ * only); replaces the same reference kernels.  token_order (optional, self-attention): as in the gather entry
+ * point above.  workspace: mindiesd_block_sparse_attention_paired_workspace_size bytes, 16-byte aligned.
+ * Returns 2 when the mask is too large for the pairing kernels (more than 2048 key blocks, or mask rows of one
+ * head beyond about 150 KiB of bits); the caller then uses the list entry points. */
+size_t mindiesd_block_sparse_attention_paired_workspace_size(int B, int N, int Sq, int Skv);
+int mindiesd_block_sparse_attention_paired_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                               int dtype, int B, int N, int Nkv, int Sq, int Skv, int D,
+                                               long long q_sb, long long q_sn, long long q_ss,
+                                               long long k_sb, long long k_sn, long long k_ss,
+                                               long long v_sb, long long v_sn, long long v_ss,
+                                               long long o_sb, long long o_sn, long long o_ss,
+                                               float scale, const signed char* mask, const int* token_order,
+                                               void* workspace, size_t ws_bytes, hipStream_t stream);
+
 /* token_order[i] (int32, S entries) = row of the original [text | image (t,h,w)] sequence that holds the
  * token at position i of RainFusion's [image in 8x8-window order | text] sequence (the index map behind
  * rearrange_with_remaining, sparse_flash_attn_rf_v2.py:137-196, 297-312). */

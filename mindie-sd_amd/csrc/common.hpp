@@ -254,6 +254,20 @@ __device__ __forceinline__ void cond_rescale_fa16(int flag, float delta, float a
   o7 = f32x4_t{o7_0, o7_1, o7_2, o7_3};
 }
 
+// Pair tables of the two-pass block-sparse attention (built by bsa_pair.hip, consumed by flash_attn_fwd.hip).
+struct BsaPairTables {
+  int* pairs;     // [BN][NP][2]
+  int* sh_idx;    // [BN][NP][KB]
+  int* sh_cnt;    // [BN][NP]
+  int* ex_idx;    // [BN][QB][KB]
+  int* ex_cnt;    // [BN][QB]
+  int* init_cnt;  // [BN][QB]
+  int NP;
+};
+size_t bsa_pair_ints(long long BN, int QB, int KB);
+bool bsa_pair_supported(int QB, int KB);
+int bsa_build_pairs(const signed char* mask, long long BN, int QB, int KB, int* ws, BsaPairTables* t, hipStream_t stream);
+
 // Lazy-rescale threshold of the online softmax, in log2 units.
 constexpr float kTau = 8.0f;
 

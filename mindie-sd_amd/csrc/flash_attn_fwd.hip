@@ -56,6 +56,11 @@ struct FaParams {
   int QB;
   const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
   const int* tok;    // GATHER instantiations: [Sq] row of q/out that holds the token at query position i
+  // two-pass block-sparse attention over paired query blocks (see bsa_pair.hip)
+  const int* pairs;     // PAIR kernel: [B * N][NP][2] query blocks of a pair (second -1: none); lists are per pair
+  int NP;
+  float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)
+  const int* init_cnt;  // second pass: [B * N][QB] key blocks the first pass covered for this query block (0: none)
   int map_mode;      // 0: consecutive query tiles of a head share an XCD; 1: linear block order
   // general mode (MODE = 1 instantiations only)
   const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
@@ -119,7 +124,12 @@ __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu
 // are fetched and output rows stored through the table.  K and V stay contiguous in the permuted order: tiles
 // gathered row by row through the same table measured 8 % slower (the block-sparse walk is bound by the L2-miss
 // path, and 2 KiB runs use it worse than 32 KiB tiles), more than the permuted copies of K and V cost.
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false>
+// INIT (block-sparse only): second pass of the paired scheme - the output rows and p.state already hold the
+// normalised result and the log-sum-exp of the key blocks covered by the first pass; the running softmax starts
+// from them (maximum = that log-sum-exp, sum = 1) instead of from nothing, and a query block without further key
+// blocks is left as it is.
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false,
+          bool INIT = false>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -216,6 +226,33 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[db][qb][r] = 0.f;
+  }
+  bool resumed = false;  // INIT: the running softmax continues the first pass (wave-uniform)
+  if constexpr (INIT) {
+    static_assert(SPARSE && C::kBM == 128 && C::kNQB == 1, "second pass: one 128-row query block per workgroup");
+    const long long qb_lin = (long long)bn * p.QB + qt;
+    const int covered = p.init_cnt[qb_lin];
+    if (covered > 0) {
+      if (p.blk_cnt[qb_lin] == 0) return;  // nothing left to add: the first pass wrote the final rows
+      resumed = true;
+      const int qrow = q0 + wave * QPW + l32;
+      const bool ok = qrow < Sq;
+      const int orow = GATHER ? p.tok[ok ? qrow : 0] : (ok ? qrow : 0);
+      const float lse2 = ok ? p.state[(long long)bn * p.Sq + qrow] : 0.f;
+      m_run[0] = lse2;
+      l_run[0] = h == 0 ? 1.f : 0.f;  // the two halves of a row add up their sums at the end
+#pragma unroll
+      for (int r = 0; r < 16; ++r) negm[0][r] = -lse2;
+      const T* orow_p = og + (long long)orow * p.o_ss;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const typename E::x4 pk = *(const typename E::x4*)(orow_p + db * 32 + 8 * g + 4 * h);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) oacc[db][0][4 * g + j] = ok ? (float)pk[j] : 0.f;
+        }
+    }
   }
 
   // ---- global -> LDS staging of one K/V tile (LDS-DMA, no registers) ------------------------------
@@ -330,7 +367,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
-  bool first = true;  // no tile has been folded into this wave's running softmax yet
+  bool first = !resumed;  // no tile has been folded into this wave's running softmax yet
 
   // One tile step: fetch the tile at next_key0 (< 0: none) into the other stage, compute on the tile
   // at key0 if this wave takes part in it.  The LDS stage is a compile-time constant (the loops
@@ -610,7 +647,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 // LDS: K stages at 0 and 32 KiB, V stages at 64 and 96 KiB, so that stage and row offsets of every read fit the
 // 16-bit offset field.  K rows are swizzled as in fa_fwd_kernel; V: 32-byte chunk c32 of row key is stored at chunk
 // c32 ^ (key & 7) - a half-wave of the transposing read covers 8 rows x 32 bytes.
-template <int DT, int NWAVES = 8>
+// PAIR: first pass of the paired block-sparse scheme (bsa_pair.hip).  The workgroup's 256 rows are two 128-row query
+// blocks that need not be neighbours (waves 0-3: p.pairs[..][0], waves 4-7: p.pairs[..][1]; -1 = no second block,
+// those waves compute on zeros and store nothing); the key tiles are the 128-key blocks of the pair's list
+// (p.blk_idx / p.blk_cnt indexed by pair) instead of the whole sequence.  Besides the normalised rows it writes
+// p.state, the log2-domain log-sum-exp the second pass resumes from.  GATHER as in fa_fwd_kernel.
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false>
 __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
@@ -627,7 +669,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int c = lane & 15;
   const int g = lane >> 4;
 
-  const int q_tiles = (p.Sq + kBM - 1) / kBM;
+  static_assert(!PAIR || NWAVES == 8, "a pair is two groups of four waves");
+  const int q_tiles = PAIR ? p.NP : (p.Sq + kBM - 1) / kBM;
   const int total = p.B * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
   const int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
@@ -637,8 +680,15 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int b = bn / p.N;
   const int n = bn - b * p.N;
   const int nkv = n / (p.N / p.Nkv);
-  const int q0 = qt * kBM;
   const int Sq = p.Sq, Skv = p.Skv;
+  // first query row of this wave; rows at or beyond row_end do not exist (tail of the sequence / of the block)
+  int row0 = qt * kBM + wave * 32, row_end = Sq;
+  if constexpr (PAIR) {
+    const int qblk = p.pairs[((long long)bn * p.NP + qt) * 2 + (wave >> 2)];
+    row0 = qblk * 128 + (wave & 3) * 32;
+    row_end = qblk < 0 ? 0 : min(Sq, qblk * 128 + 128);
+    if (qblk < 0) row0 = 0;
+  }
 
   const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
   const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
@@ -649,9 +699,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   X8 qf[2][4];
 #pragma unroll
   for (int nq = 0; nq < 2; ++nq) {
-    const int qrow = q0 + wave * 32 + nq * 16 + c;
-    const bool ok = qrow < Sq;
-    const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * g;
+    const int qrow = row0 + nq * 16 + c;
+    const bool ok = qrow < row_end;
+    const int qsrc = GATHER ? p.tok[ok ? qrow : 0] : (ok ? qrow : 0);
+    const T* src = qg + (long long)qsrc * p.q_ss + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       X8 v = *(const X8*)(src + 32 * ks);
@@ -705,7 +756,19 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
                 ((db ^ (4 * (g & 1) + (c >> 2))) << 5) + 8 * (c & 3);
 
   const int tiles = (Skv + BN - 1) / BN;
-  load_tile(0, 0);
+  // PAIR: the ids of the list are fetched with scalar loads two tiles ahead of their use
+  int l_n = 0, id_a = -1, id_b = -1;  // id_a: the tile being computed (already requested), id_b: the one after it
+  const int* l_ptr = nullptr;
+  if constexpr (PAIR) {
+    const long long pair_lin = (long long)bn * p.NP + qt;
+    l_ptr = p.blk_idx + pair_lin * p.kb_stride;
+    l_n = __builtin_amdgcn_readfirstlane(p.blk_cnt[pair_lin]);
+    if (l_n > 0) id_a = __builtin_amdgcn_readfirstlane(l_ptr[0]);
+    if (l_n > 1) id_b = __builtin_amdgcn_readfirstlane(l_ptr[1]);
+    if (l_n > 0) load_tile(id_a * BN, 0);
+  } else {
+    load_tile(0, 0);
+  }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   bool first = true;
@@ -835,9 +898,21 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next tile has landed
     __syncthreads();
   };
-  for (int t = 0; t < tiles; t += 2) {
-    tile_step(std::integral_constant<int, 0>{}, t * BN, t + 1 < tiles ? (t + 1) * BN : -1);
-    if (t + 1 < tiles) tile_step(std::integral_constant<int, 1>{}, (t + 1) * BN, t + 2 < tiles ? (t + 2) * BN : -1);
+  if constexpr (PAIR) {
+    for (int pos = 0; pos < l_n; pos += 2) {
+      const int id_c = pos + 2 < l_n ? __builtin_amdgcn_readfirstlane(l_ptr[pos + 2]) : -1;
+      tile_step(std::integral_constant<int, 0>{}, id_a * BN, id_b >= 0 ? id_b * BN : -1);
+      if (id_b < 0) break;
+      const int id_d = pos + 3 < l_n ? __builtin_amdgcn_readfirstlane(l_ptr[pos + 3]) : -1;
+      tile_step(std::integral_constant<int, 1>{}, id_b * BN, id_c >= 0 ? id_c * BN : -1);
+      id_a = id_c;
+      id_b = id_d;
+    }
+  } else {
+    for (int t = 0; t < tiles; t += 2) {
+      tile_step(std::integral_constant<int, 0>{}, t * BN, t + 1 < tiles ? (t + 1) * BN : -1);
+      if (t + 1 < tiles) tile_step(std::integral_constant<int, 1>{}, (t + 1) * BN, t + 2 < tiles ? (t + 2) * BN : -1);
+    }
   }
 
   // ---- epilogue: normalise, transpose the wave's 32 query rows through LDS, coalesced store --------------------
@@ -846,10 +921,14 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   for (int nq = 0; nq < 2; ++nq) {
     const float l_tot = quarter_sum(l_run[nq]);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int qrow_l = q0 + wave * 32 + nq * 16 + c;
-    if (p.lse && g == 0 && qrow_l < Sq)
-      p.lse[((long long)b * p.N + n) * p.Sq + qrow_l] =
+    const int qrow_l = row0 + nq * 16 + c;
+    if (p.lse && g == 0 && qrow_l < row_end)
+      p.lse[((long long)b * p.N + n) * p.Sq + (GATHER ? p.tok[qrow_l] : qrow_l)] =
           l_tot > 0.f ? -negm[nq][0] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
+    if constexpr (PAIR) {
+      if (g == 0 && qrow_l < row_end)
+        p.state[((long long)b * p.N + n) * p.Sq + qrow_l] = l_tot > 0.f ? -negm[nq][0] + __log2f(l_tot) : -INFINITY;
+    }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
       typename E::x4 pk;
@@ -863,32 +942,34 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   for (int i = 0; i < 32 * 16 / 64; ++i) {
     const int ch = i * 64 + lane;
     const int row = ch >> 4, c16 = ch & 15;
-    const int qrow = q0 + wave * 32 + row;
+    const int qrow = row0 + row;
     const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16);
     const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16 + 8);
-    if (qrow < Sq) {
+    if (qrow < row_end) {
       i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
-      *(i32x4_t*)(og + (long long)qrow * p.o_ss + c16 * 8) = v;
+      const int orow = GATHER ? p.tok[qrow] : qrow;
+      *(i32x4_t*)(og + (long long)orow * p.o_ss + c16 * 8) = v;
     }
   }
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int NWAVES = 8>
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false>
 static int launch_fa16(const FaParams& p, hipStream_t stream) {
   constexpr int kLds = 4 * 128 * 256;  // two K and two V stages of 128 keys
-  auto kern = fa_fwd16_kernel<DT, NWAVES>;
+  auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const int total = p.B * p.N * ((p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
+  const int total = p.B * p.N * (PAIR ? p.NP : (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
   hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
-template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false>
+template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false,
+          bool INIT = false>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
-  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE, GATHER>;
+  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE, GATHER, INIT>;
   // per device and idempotent, so it is simply repeated on every launch
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
     return MSD_ERR_LAUNCH;
@@ -994,6 +1075,58 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
   p.QB = (S + 127) / 128;
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, true>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, true>(p, stream);
+}
+
+// Block-sparse attention driven by the int8 mask itself, in two passes over paired query blocks (bsa_pair.hip):
+// pairing + lists, then the key blocks both partners of a pair selected (256-row workgroups, the dense kernel's
+// inner loop), then what only one of them selected, continuing the running softmax.  Same result as
+// mindiesd_block_sparse_attention_fwd on the lists of the mask up to the order of accumulation.
+size_t mindiesd_block_sparse_attention_paired_workspace_size(int B, int N, int Sq, int Skv) {
+  if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return 0;
+  const long long BN = (long long)B * N;
+  const int QB = (Sq + 127) / 128, KB = (Skv + 127) / 128;
+  return bsa_pair_ints(BN, QB, KB) * sizeof(int) + (size_t)BN * Sq * sizeof(float);
+}
+
+int mindiesd_block_sparse_attention_paired_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                               int dtype, int B, int N, int Nkv, int Sq, int Skv, int D,
+                                               long long q_sb, long long q_sn, long long q_ss, long long k_sb,
+                                               long long k_sn, long long k_ss, long long v_sb, long long v_sn,
+                                               long long v_ss, long long o_sb, long long o_sn, long long o_ss,
+                                               float scale, const signed char* mask, const int* token_order,
+                                               void* workspace, size_t ws_bytes, hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (!mask || !workspace || ((uintptr_t)workspace & 15)) return MSD_ERR_BAD_ARG;
+  if (token_order && Sq != Skv) return MSD_ERR_BAD_ARG;
+  const int QB = (Sq + 127) / 128, KB = (Skv + 127) / 128;
+  if (!bsa_pair_supported(QB, KB)) return MSD_ERR_UNSUPPORTED;
+  if (ws_bytes < mindiesd_block_sparse_attention_paired_workspace_size(B, N, Sq, Skv)) return MSD_ERR_WORKSPACE;
+  const long long BN = (long long)B * N;
+  BsaPairTables t;
+  float* state = (float*)workspace;  // first, so that it stays 16-byte aligned
+  rc = bsa_build_pairs(mask, BN, QB, KB, (int*)(state + BN * Sq), &t, stream);
+  if (rc != MSD_OK) return rc;
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  p.tok = token_order;
+  p.QB = QB;
+  p.state = state;
+  // pass 1: one workgroup per pair over the shared list
+  p.pairs = t.pairs; p.NP = t.NP;
+  p.blk_idx = t.sh_idx; p.blk_cnt = t.sh_cnt; p.kb_stride = KB;
+  if (dtype == MSD_DTYPE_BF16)
+    rc = token_order ? launch_fa16<MSD_DTYPE_BF16, 8, true, true>(p, stream) : launch_fa16<MSD_DTYPE_BF16, 8, true, false>(p, stream);
+  else
+    rc = token_order ? launch_fa16<MSD_DTYPE_F16, 8, true, true>(p, stream) : launch_fa16<MSD_DTYPE_F16, 8, true, false>(p, stream);
+  if (rc != MSD_OK) return rc;
+  // pass 2: one workgroup per query block over its exclusive list, resuming from pass 1
+  p.blk_idx = t.ex_idx; p.blk_cnt = t.ex_cnt; p.init_cnt = t.init_cnt;
+  if (dtype == MSD_DTYPE_BF16)
+    return token_order ? launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, true, true>(p, stream)
+                       : launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, false, true>(p, stream);
+  return token_order ? launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, true, true>(p, stream)
+                     : launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, false, true>(p, stream);
 }
 
 int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,

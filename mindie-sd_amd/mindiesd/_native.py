@@ -37,6 +37,9 @@ SIGNATURES = {
     "mindiesd_lpt_order": (c_int, [c_p, c_p, c_int, c_int, c_p]),
     "mindiesd_block_sparse_attention_gather_fwd": (c_int, [c_p] * 5 + [c_int] * 6 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_p,
                                                                                             c_p]),
+    "mindiesd_block_sparse_attention_paired_workspace_size": (c_sz, [c_int] * 4),
+    "mindiesd_block_sparse_attention_paired_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_p, c_p, c_sz,
+                                                                                          c_p]),
     "mindiesd_rf_token_order": (c_int, [c_p] + [c_int] * 5 + [c_p]),
     "mindiesd_fa_block_quant": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_int, c_f, c_int, c_p]),
     "mindiesd_fa_rot_block_quant": (c_int, [c_p, c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_f, c_int, c_p]),

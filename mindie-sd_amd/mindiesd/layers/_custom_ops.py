@@ -102,9 +102,8 @@ def _block_sparse_attention_impl(query, key, value, block_sparse_mask=None, bloc
         q4, k4, v4, layout = query, key, value, "BNSD"
         _check_lengths(actual_seq_lengths, query.shape[2], "block_sparse_attention")
         _check_lengths(actual_seq_lengths_kv, key.shape[2], "block_sparse_attention")
-    idx, cnt = rf.mask_to_lists(block_sparse_mask)
     want_lse = softmax_lse_flag != 0
-    res = rf.block_sparse_attention_lists(q4, k4, v4, idx, cnt, scale_value, layout, return_lse=want_lse)
+    res = rf.block_sparse_attention_mask(q4, k4, v4, block_sparse_mask, scale_value, layout, return_lse=want_lse)
     out, lse = res if want_lse else (res, None)
     if q_input_layout == "TND":
         out = out.reshape(query.shape)
@@ -159,9 +158,19 @@ def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blo
         b, n = query.shape[0], query.shape[1]
     if select_idx.dim() != 3 or select_idx.shape[1] != n or tuple(select_num_idx.shape) != tuple(select_idx.shape[:2]):
         raise RuntimeError("select_idx must be [q_blocks, N, kv_blocks] and select_num_idx [q_blocks, N]")
-    idx = select_idx.permute(1, 0, 2).to(torch.int32).unsqueeze(0).expand(b, -1, -1, -1).contiguous()
-    cnt = select_num_idx.permute(1, 0).to(torch.int32).unsqueeze(0).expand(b, -1, -1).contiguous()
-    out, lse = rf.block_sparse_attention_lists(q4, k4, v4, idx, cnt, scale, layout, return_lse=True)
+    # The selection as an int8 mask: entry j of a row counts if j < select_num_idx and the id names a key block
+    # (ids outside [0, kv_blocks) and entries past the count are dropped, so a malformed list cannot make the
+    # kernel read outside its tables).  The mask form runs the paired two-pass kernel.
+    skv = k4.shape[2] if layout == "BNSD" else k4.shape[1]
+    kb = (skv + 127) // 128
+    sel = select_idx.permute(1, 0, 2).to(torch.int64)                               # [N, qb, width]
+    num = select_num_idx.permute(1, 0).to(torch.int64).unsqueeze(-1)                # [N, qb, 1]
+    pos = torch.arange(sel.shape[-1], device=sel.device).view(1, 1, -1)
+    valid = (pos < num) & (sel >= 0) & (sel < kb)
+    mask = torch.zeros((n, sel.shape[1], kb + 1), dtype=torch.int8, device=sel.device)
+    mask.scatter_(2, torch.where(valid, sel + 1, torch.zeros_like(sel)), 1)         # column 0 takes the dropped ones
+    mask = mask[:, :, 1:].unsqueeze(0).expand(b, -1, -1, -1).contiguous()
+    out, lse = rf.block_sparse_attention_mask(q4, k4, v4, mask, scale, layout, return_lse=True)
     if q_input_layout == "TND":
         out = out.reshape(query.shape)
         lse_out = torch.zeros(query.shape, dtype=query.dtype, device=query.device)

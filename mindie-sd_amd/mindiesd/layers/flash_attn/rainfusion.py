@@ -324,6 +324,49 @@ def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, lay
     return (out, lse) if return_lse else out
 
 
+def block_sparse_attention_mask(query, key, value, block_sparse_mask, scale, layout="BNSD", return_lse=False,
+                                order=None):
+    """Attention of every 128-row query block over the key blocks its mask row selects
+    (``block_sparse_mask`` int8/bool [B, N, qb, kb], non-zero = attend; an all-zero row yields zeros).
+    Runs the two-pass kernel over paired query blocks (query blocks with similar mask rows share their K/V
+    tiles); masks too large for the pairing kernels go through the block lists.  ``order`` as in
+    :func:`block_sparse_attention_lists`."""
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        _check_gpu16(t, name)
+    q, k, v = _aligned(query), _aligned(key), _aligned(value)
+    b, n, sq = _dims(q, layout)
+    _, nkv, skv = _dims(k, layout)
+    if k.shape != v.shape or k.shape[0] != b or n % nkv != 0 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ParametersInvalid("Inconsistent query/key/value shapes or dtypes.")
+    qb, kb = (sq + BLOCK - 1) // BLOCK, (skv + BLOCK - 1) // BLOCK
+    if block_sparse_mask.dim() != 4 or tuple(block_sparse_mask.shape) != (b, n, qb, kb) or not block_sparse_mask.is_cuda:
+        raise ParametersInvalid(f"block_sparse_mask must be a GPU tensor [B, N, {qb}, {kb}], but got "
+                                f"{tuple(block_sparse_mask.shape)}.")
+    if order is not None and (order.dtype != torch.int32 or order.dim() != 1 or order.shape[0] != sq or skv != sq
+                              or not order.is_contiguous() or order.device != q.device):
+        raise ParametersInvalid(f"order must be a contiguous int32 [{sq}] tensor on the inputs' device "
+                                "(self-attention only).")
+    m8 = block_sparse_mask if block_sparse_mask.dtype == torch.int8 else block_sparse_mask.to(torch.int8)
+    m8 = m8.contiguous()
+    lib = _native.lib()
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, n, sq), dtype=torch.float32, device=q.device) if return_lse else None
+    ws_bytes = lib.mindiesd_block_sparse_attention_paired_workspace_size(b, n, sq, skv)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.mindiesd_block_sparse_attention_paired_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
+            _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1],
+            *_strides_bns(q, layout), *_strides_bns(k, layout), *_strides_bns(v, layout), *_strides_bns(out, layout),
+            float(scale), m8.data_ptr(), order.data_ptr() if order is not None else None, ws.data_ptr(), ws_bytes,
+            _native.stream_ptr(q.device))
+    if rc == 2 and q.shape[-1] == HEAD_DIM:  # mask too large for the pairing kernels
+        idx, cnt = mask_to_lists(m8)
+        return block_sparse_attention_lists(q, k, v, idx, cnt, scale, layout, return_lse, order)
+    _native.check(rc, "mindiesd_block_sparse_attention_paired_fwd")
+    return (out, lse) if return_lse else out
+
+
 def mask_to_lists(block_sparse_mask):
     """int8/bool [B, N, qb, kb] (non-zero = attend) -> (blk_idx int32 [B,N,qb,kb], blk_cnt int32 [B,N,qb])."""
     if block_sparse_mask.dim() != 4 or not block_sparse_mask.is_cuda:
@@ -364,8 +407,7 @@ def rain_fusion_attention_v3(query, key, value, block_sparse_mask, scale=None, h
     _check_layout(input_layout)
     if sparse_size != BLOCK:
         raise ParametersInvalid(f"sparse_size only supports {BLOCK}, but got {sparse_size}.")
-    idx, cnt = mask_to_lists(block_sparse_mask)
-    return block_sparse_attention_lists(query, key, value, idx, cnt, scale, input_layout)
+    return block_sparse_attention_mask(query, key, value, block_sparse_mask, scale, input_layout)
 
 
 def bsa_sparse_attention_v3(q, k, v, latent_shape_q, latent_shape_k=None, txt_len=0, pool_size=128, sparsity=0.5,
@@ -401,12 +443,11 @@ def bsa_sparse_attention_v3(q, k, v, latent_shape_q, latent_shape_k=None, txt_le
         shape = (3 * b, n, nb, q.shape[-1]) if input_layout == "BNSD" else (3 * b, nb, n, q.shape[-1])
         pool = torch.empty(shape, dtype=q.dtype, device=q.device)
         _run_rearrange([q, k, v], [None, k_, v_], pool, input_layout, grid, txt_len, 0)
-        new_mask, idx, cnt, _, _ = _block_mask(pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout,
-                                               protect_first_frame, keep_diagonal, True, True, False)
+        new_mask, _, _, _, _ = _block_mask(pool, txt_len, sparsity, scale, pool_size, latent_shape_q, input_layout,
+                                           protect_first_frame, keep_diagonal, True, False, False)
     else:
         _run_rearrange([k, v], [k_, v_], None, input_layout, grid, txt_len, 0)
         new_mask = cached_mask
-        idx, cnt = mask_to_lists(cached_mask)
-    out = block_sparse_attention_lists(q, k_, v_, idx, cnt, scale, input_layout,
-                                       order=token_order(grid, txt_len, q.device))
+    out = block_sparse_attention_mask(q, k_, v_, new_mask, scale, input_layout,
+                                      order=token_order(grid, txt_len, q.device))
     return out, new_mask
