@@ -56,7 +56,8 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
  *   causal != 0: key j is visible to query i iff j <= i + (Skv - Sq), the lower triangle aligned to the
  *     bottom-right corner (the vendor kernel's sparse_mode = 3, attention_forward_varlen.py:134-136).
  *   mask != NULL: boolean mask, one byte per (query, key), non-zero = attend, keys contiguous, element
- *     strides m_sb / m_sn (0 = broadcast over batch / heads) and m_sq.  Replaces the atten_mask argument
+ *     strides m_sb / m_sn (0 = broadcast over batch / heads) and m_sq (>= Skv, or 0 = one row for all queries).
+ *     Replaces the atten_mask argument
  *     of the fused wrappers (prompt_flash_attn.py:46-52, fused_attn_score.py:46-52; they pass the
  *     inverted mask, this entry point takes it as the caller of attention_forward gives it).
  * A query row without any visible key gives zeros (and lse = -inf). */
@@ -69,9 +70,6 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
                                          float scale, const int* seq_meta, int causal,
                                          const unsigned char* mask, long long m_sb, long long m_sn, long long m_sq,
                                          hipStream_t stream);
-
-/* Benchmark hook: selects one of the compiled dense kernel variants (0 = default). */
-void mindiesd_set_dense_variant(int variant);
 
 /* ---- block-sparse attention ------------------------------------------------------------------------
  * Query block i (128 rows) of (b, n) attends to the 128-key blocks blk_idx[b][n][i][0 .. blk_cnt[b][n][i])
@@ -105,6 +103,23 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
                                                long long o_sb, long long o_sn, long long o_ss,
                                                float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
                                                const int* token_order, hipStream_t stream);
+
+/* Block-sparse attention with per-sequence lengths (the actual_seq_lengths / actual_seq_lengths_kv arguments of
+ * aclnnBlockSparseAttention, csrc/plugin/block_sparse_attention.cpp:42-66, 100-121): seq_meta int32 [B][4] =
+ * {first query token, query count, first key token, key count} as in mindiesd_flash_attention_general_fwd.  Layout
+ * "TND": packed [T][N][128] tensors, batch strides 0; layout "BNSD" with shorter sequences: ordinary batch strides,
+ * first tokens 0.  Sq / Skv = the longest counts; blk_idx / blk_cnt are per (batch, head, query block) of that
+ * length.  lse (optional): [B][N][Sq], or with lse_token_major != 0 [T][N].  Query rows past a sequence's count
+ * are not written.  causal != 0: key j visible to query i iff j <= i + (key count - query count). */
+int mindiesd_block_sparse_attention_general_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                                int dtype, int B, int N, int Nkv, int Sq, int Skv, int D,
+                                                long long q_sb, long long q_sn, long long q_ss,
+                                                long long k_sb, long long k_sn, long long k_ss,
+                                                long long v_sb, long long v_sn, long long v_ss,
+                                                long long o_sb, long long o_sn, long long o_ss,
+                                                float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                                const int* seq_meta, int lse_token_major, int causal,
+                                                hipStream_t stream);
 
 /* Block-sparse attention driven by the int8 mask itself (mask [B][N][ceil(Sq/128)][ceil(Skv/128)], non-zero =
  * attend), in two passes over PAIRED query blocks: query blocks of a head whose mask rows overlap most are paired
@@ -204,9 +219,6 @@ int mindiesd_rf_block_mask(const void* q_pool, const void* k_pool, int dtype, in
  * mindiesd_block_sparse_attention_fwd consumes). */
 int mindiesd_mask_to_index(const signed char* mask, int BN, int QB, int KB, int* blk_idx, int* blk_cnt,
                            int kb_stride, hipStream_t stream);
-
-/* Dispatch order for the block-sparse kernel: query blocks sorted by descending block count. */
-int mindiesd_lpt_order(const int* blk_cnt, int* order, int total, int max_cnt, hipStream_t stream);
 
 /* ---- FP8 attention -----------------------------------------------------------------------------------
  * Block quantisation of one attention operand: x [B][N][S][128] 16-bit (strided) ->

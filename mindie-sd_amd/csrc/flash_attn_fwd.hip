@@ -61,10 +61,10 @@ struct FaParams {
   int NP;
   float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)
   const int* init_cnt;  // second pass: [B * N][QB] key blocks the first pass covered for this query block (0: none)
-  int map_mode;      // 0: consecutive query tiles of a head share an XCD; 1: linear block order
   // general mode (MODE = 1 instantiations only)
   const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
                               // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count
+  int lse_token_major;        // with seq_meta: lse is [tokens][N] (index (first query token + row) * N + head)
   int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
   const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
   long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
   const int total = p.B * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
-  int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
+  int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (SPARSE && p.order) {  // caller's work order: workgroup i takes entry i of the table
     if ((int)blockIdx.x >= total) return;
     work = p.order[blockIdx.x];
@@ -600,7 +600,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int qrow_l = q0 + wave * QPW + qb * 32 + l32;
     if (p.lse && h == 0 && qrow_l < Sq) {
-      const long long li = ((long long)b * p.N + n) * p.Sq + (GATHER ? p.tok[qrow_l] : qrow_l);
+      long long li = ((long long)b * p.N + n) * p.Sq + (GATHER ? p.tok[qrow_l] : qrow_l);
+      if (MODE && p.seq_meta && p.lse_token_major) li = ((long long)p.seq_meta[4 * b] + qrow_l) * p.N + n;
       p.lse[li] = l_tot > 0.f ? m_run[qb] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
     }
 #pragma unroll
@@ -673,7 +674,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int q_tiles = PAIR ? p.NP : (p.Sq + kBM - 1) / kBM;
   const int total = p.B * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
-  const int work = p.map_mode == 0 ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : (int)blockIdx.x;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
   const int bn = work / q_tiles;
   const int qt = work - bn * q_tiles;
@@ -986,18 +987,6 @@ using namespace msd;
 
 extern "C" {
 
-// Tuning hook used by benchmark sweeps: selects the dense kernel variant
-// (0, default: fa_fwd16_kernel, 8 waves x 32 rows, 128-key tiles on the 16x16x32 matrix instruction;
-//  4: the same tile shape on the 32x32x16 instruction (fa_fwd_kernel), operand reads scheduled one step ahead;
-//  1: 4 waves x 32 rows, 64-key tiles, compiler scheduling; 2: as 4 with compiler scheduling;
-//  3: as 1 with scheduled operand reads).
-static int g_dense_variant = 0;
-static int g_map_mode = 0;  // bits 8.. of the variant: tile order (0 = per-XCD chunks, 1 = linear)
-void mindiesd_set_dense_variant(int v) {
-  g_dense_variant = v & 0xff;
-  g_map_mode = (v >> 8) & 0xff;
-}
-
 static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
                         int Nkv, int Sq, int Skv, int D, const long long* st, float scale) {
   if (!q || !k || !v || !out) return MSD_ERR_BAD_ARG;
@@ -1041,14 +1030,7 @@ int mindiesd_block_sparse_attention_fwd(const void* q, const void* k, const void
   if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.order = order;
-  p.map_mode = g_map_mode;
   p.QB = (Sq + 127) / 128;
-  if (g_dense_variant == 7) {
-    // tuning hook: two query blocks per workgroup walking the merge of their lists (128-key tiles).
-    // Pays off only when neighbouring query blocks select mostly the same key blocks.
-    if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, true, 1>(p, stream);
-    return launch_fa<MSD_DTYPE_F16, 8, 32, 128, true, 1>(p, stream);
-  }
   // one query block per workgroup, 64-key sub-tiles, two workgroups per CU
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
@@ -1071,7 +1053,6 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
   if (!blk_idx || !blk_cnt || kb_stride <= 0 || !token_order) return MSD_ERR_BAD_ARG;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, S, S, st, scale);
   p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride; p.tok = token_order;
-  p.map_mode = g_map_mode;
   p.QB = (S + 127) / 128;
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, true>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, true>(p, stream);
@@ -1138,17 +1119,7 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
   if (rc != MSD_OK) return rc;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
-  p.map_mode = g_map_mode;
-  if (dtype == MSD_DTYPE_BF16) {
-    switch (g_dense_variant) {
-      case 1: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 0>(p, stream);
-      case 2: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 0>(p, stream);
-      case 3: return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1>(p, stream);
-      case 4: return launch_fa<MSD_DTYPE_BF16, 8, 32, 128, false, 1>(p, stream);
-      case 5: return launch_fa16<MSD_DTYPE_BF16, 4>(p, stream);
-      default: return launch_fa16<MSD_DTYPE_BF16>(p, stream);
-    }
-  }
+  if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16>(p, stream);
   return launch_fa16<MSD_DTYPE_F16>(p, stream);
 }
 
@@ -1166,13 +1137,38 @@ int mindiesd_ada_block_sparse_attention_fwd(const void* q, const void* k, const 
   if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
   FaParams p = make_params(q, k, v, out, nullptr, B, N, Nkv, S, S, st, scale);
   p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride;
-  p.map_mode = g_map_mode;
   p.QB = (S + 127) / 128;
   p.causal = causal ? 1 : 0;
   if (!causal) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1>(p, stream);
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1>(p, stream);
   }
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 1>(p, stream);
+}
+
+// Block-sparse attention with per-sequence lengths: seq_meta [B][4] = {first query token, query count, first key
+// token, key count} as in mindiesd_flash_attention_general_fwd.  With batch strides 0 the tensors are packed
+// (token, head, dim) arrays; with ordinary batch strides and first tokens 0 it gives every batch entry its own
+// length inside [B][N][S][128] tensors.  Sq / Skv are the longest counts; the lists are per (batch, head, query
+// block of that length).  Query rows past a sequence's count are not written.
+int mindiesd_block_sparse_attention_general_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                                                int dtype, int B, int N, int Nkv, int Sq, int Skv, int D,
+                                                long long q_sb, long long q_sn, long long q_ss, long long k_sb,
+                                                long long k_sn, long long k_ss, long long v_sb, long long v_sn,
+                                                long long v_ss, long long o_sb, long long o_sn, long long o_ss,
+                                                float scale, const int* blk_idx, const int* blk_cnt, int kb_stride,
+                                                const int* seq_meta, int lse_token_major, int causal,
+                                                hipStream_t stream) {
+  const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  if (rc != MSD_OK) return rc;
+  if (!blk_idx || !blk_cnt || kb_stride <= 0) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  p.blk_idx = blk_idx; p.blk_cnt = blk_cnt; p.kb_stride = kb_stride;
+  p.QB = (Sq + 127) / 128;
+  p.seq_meta = seq_meta; p.lse_token_major = lse_token_major ? 1 : 0;
+  p.causal = causal ? 1 : 0;
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 1>(p, stream);
 }
@@ -1191,9 +1187,9 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
   if (rc != MSD_OK) return rc;
   if (seq_meta && (mask || lse)) return MSD_ERR_UNSUPPORTED;  // packed sequences: neither mask nor lse layout defined
-  if (mask && (m_sb < 0 || m_sn < 0 || m_sq < Skv)) return MSD_ERR_BAD_ARG;
+  // m_sq == 0: one mask row shared by all queries (a key-padding mask expanded over the query dimension)
+  if (mask && (m_sb < 0 || m_sn < 0 || (m_sq != 0 && m_sq < Skv))) return MSD_ERR_BAD_ARG;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
-  p.map_mode = g_map_mode;
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);

@@ -636,6 +636,7 @@ int mindiesd_fa_block_quant(const void* x, void* q, float* scale, int dtype, int
   if (block_size != 128 && block_size != 256 && block_size != 512) return MSD_ERR_BAD_ARG;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
   if (((uintptr_t)x & 15) || ((uintptr_t)q & 7) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
+  if ((long long)B * N > 65535) return MSD_ERR_UNSUPPORTED;  // grid.y
   dim3 grid((S + block_size - 1) / block_size, B * N);
   if (block_size == 128) {
     if (dtype == MSD_DTYPE_BF16)

@@ -329,25 +329,6 @@ __global__ __launch_bounds__(256) void mask_to_index_kernel(const signed char* m
   if (tid == 0) blk_cnt[row_lin] = total;
 }
 
-// Work order for the block-sparse attention kernel: query blocks sorted by descending number of
-// selected key blocks (longest first), via a counting sort on the counts.  Single workgroup.
-__global__ __launch_bounds__(1024) void lpt_order_kernel(const int* blk_cnt, int* order, int total, int max_cnt) {
-  extern __shared__ int bins[];  // max_cnt + 2 entries
-  for (int i = threadIdx.x; i < max_cnt + 2; i += blockDim.x) bins[i] = 0;
-  __syncthreads();
-  for (int i = threadIdx.x; i < total; i += blockDim.x) atomicAdd(&bins[max_cnt - min(blk_cnt[i], max_cnt) + 1], 1);
-  __syncthreads();
-  if (threadIdx.x == 0)
-    for (int i = 1; i < max_cnt + 2; ++i) bins[i] += bins[i - 1];
-  __syncthreads();
-  // positions inside a bin are handed out by atomics: the order inside equal counts is arbitrary,
-  // which only affects scheduling, never results
-  for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int bin = max_cnt - min(blk_cnt[i], max_cnt);
-    order[atomicAdd(&bins[bin], 1)] = i;
-  }
-}
-
 }  // namespace msd
 
 using namespace msd;
@@ -428,13 +409,6 @@ int mindiesd_mask_to_index(const signed char* mask, int BN, int QB, int KB, int*
   if (!mask || !blk_idx || !blk_cnt || BN <= 0 || QB <= 0 || KB <= 0 || kb_stride < KB) return MSD_ERR_BAD_ARG;
   hipLaunchKernelGGL(mask_to_index_kernel, dim3(QB, BN), dim3(256), 0, stream, mask, blk_idx, blk_cnt, QB, KB,
                      kb_stride);
-  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
-}
-
-int mindiesd_lpt_order(const int* blk_cnt, int* order, int total, int max_cnt, hipStream_t stream) {
-  if (!blk_cnt || !order || total <= 0 || max_cnt < 0 || max_cnt > 8192) return MSD_ERR_BAD_ARG;
-  hipLaunchKernelGGL(lpt_order_kernel, dim3(1), dim3(1024), (max_cnt + 2) * sizeof(int), stream, blk_cnt, order,
-                     total, max_cnt);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 

@@ -29,17 +29,17 @@ SIGNATURES = {
     "mindiesd_sbe_scores_workspace_size": (c_sz, [c_int, c_int]),
     "mindiesd_sbe_scores": (c_int, [c_p, c_p, c_p] + [c_int] * 6 + [c_ll] * 6 + [c_f, c_int, c_p, c_sz, c_p]),
     "mindiesd_sbe_select": (c_int, [c_p, c_p, c_p] + [c_int] * 3 + [c_f, c_f, c_int, c_int, c_int, c_p]),
-    "mindiesd_set_dense_variant": (None, [c_int]),
     "mindiesd_block_sparse_attention_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_p, c_p]),
     "mindiesd_rf_rearrange_pool": (c_int, [c_p] * 7 + [c_int] * 5 + [c_ll] * 10 + [c_int] * 6 + [c_p]),
     "mindiesd_rf_block_mask": (c_int, [c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_f] + [c_int] * 4 + [c_p] * 3 + [c_int, c_p, c_p, c_p]),
     "mindiesd_mask_to_index": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_int, c_p]),
-    "mindiesd_lpt_order": (c_int, [c_p, c_p, c_int, c_int, c_p]),
     "mindiesd_block_sparse_attention_gather_fwd": (c_int, [c_p] * 5 + [c_int] * 6 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_p,
                                                                                             c_p]),
     "mindiesd_block_sparse_attention_paired_workspace_size": (c_sz, [c_int] * 4),
     "mindiesd_block_sparse_attention_paired_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_p, c_p, c_sz,
                                                                                           c_p]),
+    "mindiesd_block_sparse_attention_general_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_p,
+                                                                                           c_int, c_int, c_p]),
     "mindiesd_rf_token_order": (c_int, [c_p] + [c_int] * 5 + [c_p]),
     "mindiesd_fa_block_quant": (c_int, [c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_int, c_f, c_int, c_p]),
     "mindiesd_fa_rot_block_quant": (c_int, [c_p, c_p, c_p, c_p] + [c_int] * 5 + [c_ll] * 3 + [c_f, c_int, c_p]),

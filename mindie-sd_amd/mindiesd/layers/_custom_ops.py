@@ -3,7 +3,10 @@
 Schemas of ``rainfusionattention`` and ``block_sparse_attention`` are the reference's
 (csrc/plugin/register_ops.cpp:41-45, :62-67), likewise ``ada_block_sparse_attention`` and
 ``sparse_block_estimate`` (:46-59); the wrappers mirror mindiesd/layers/_custom_ops.py
-(:124-189, :204-305, :330-390).  ``flash_attention_fwd`` is the dense kernel as an op."""
+(:124-189, :204-305, :330-390).  New ops of this build (no counterpart in the reference, which reaches the
+vendor kernels through torch_npu): ``flash_attention_fwd`` (dense kernel), ``fa_block_quant``, ``fp8_attention_fwd``,
+``mxfp8_gemm_swiglu`` and ``rf_block_mask``; each has a fake implementation, so that ``torch.compile`` traces
+through the FP8 / MXFP8 / RainFusion path the way the reference's ops do (mindiesd/layers/register_ops.py:90-128)."""
 from typing import List, Optional, Tuple
 
 import torch
@@ -38,6 +41,20 @@ register_ops.define_op(
 register_ops.define_op(
     "flash_attention_fwd",
     "(Tensor query, Tensor key, Tensor value, float scale_value=1.0, str input_layout='BNSD') -> (Tensor, Tensor)")
+register_ops.define_op(
+    "fa_block_quant",
+    "(Tensor x, int block_size=128, str input_layout='BNSD') -> (Tensor, Tensor)")
+register_ops.define_op(
+    "fp8_attention_fwd",
+    "(Tensor query, Tensor key, Tensor value, float scale_value=1.0, str input_layout='BNSD', Tensor? q_rot=None, "
+    "Tensor? k_rot=None, str recipe='amax') -> Tensor")
+register_ops.define_op(
+    "mxfp8_gemm_swiglu",
+    "(Tensor x, Tensor weight, Tensor weight_scale, Tensor? bias=None, bool swiglu=True) -> Tensor")
+register_ops.define_op(
+    "rf_block_mask",
+    "(Tensor qkv_pool, int txt_len, float sparsity, float scale, int[] latent_shape, str input_layout='BNSD', "
+    "bool protect_first_frame=True, bool keep_diagonal=False) -> Tensor")
 
 
 def _tnd_as_bsnd(t, seq_lens, what):
@@ -49,6 +66,16 @@ def _tnd_as_bsnd(t, seq_lens, what):
     if len(set(seq_lens)) != 1 or seq_lens[0] * len(seq_lens) != t.shape[0]:
         raise RuntimeError(f"{what}: TND layout supports equal sequence lengths that sum to T only")
     return t.reshape(len(seq_lens), seq_lens[0], t.shape[1], t.shape[2])
+
+
+def _varlen(what, *args, **kwargs):
+    """rf.block_sparse_attention_varlen with argument errors as RuntimeError (what TORCH_CHECK gives in the
+    reference's plugin)."""
+    from .flash_attn import rainfusion as rf
+    try:
+        return rf.block_sparse_attention_varlen(*args, **kwargs)
+    except ParametersInvalid as e:
+        raise RuntimeError(f"{what}: {e}") from e
 
 
 def _check_lengths(actual, s, what):
@@ -93,16 +120,34 @@ def _block_sparse_attention_impl(query, key, value, block_sparse_mask=None, bloc
         raise RuntimeError(f"block_sparse_attention: block_shape only supports [128, 128], got {list(block_shape)}")
     if block_sparse_mask is None:
         raise RuntimeError("block_sparse_attention: block_sparse_mask is required")
+    want_lse = softmax_lse_flag != 0
+    lens_q = [int(x) for x in actual_seq_lengths] if actual_seq_lengths is not None else None
+    lens_kv = [int(x) for x in actual_seq_lengths_kv] if actual_seq_lengths_kv is not None else None
     if q_input_layout == "TND":
-        q4 = _tnd_as_bsnd(query, list(actual_seq_lengths), "block_sparse_attention")
-        k4 = _tnd_as_bsnd(key, list(actual_seq_lengths_kv), "block_sparse_attention")
-        v4 = _tnd_as_bsnd(value, list(actual_seq_lengths_kv), "block_sparse_attention")
+        equal = len(set(lens_q)) == 1 and len(set(lens_kv)) == 1 and len(lens_q) == len(lens_kv)
+        if not equal:  # sequences of different lengths packed one after the other
+            res = _varlen("block_sparse_attention", query, key, value, block_sparse_mask, scale_value, lens_q, lens_kv,
+                          "TND", return_lse=want_lse)
+            out, lse = res if want_lse else (res, None)
+            lse_out = lse.unsqueeze(-1) if want_lse else torch.empty(
+                (query.shape[0], query.shape[1], 1), dtype=torch.float32, device=query.device)
+            return out, lse_out
+        q4 = _tnd_as_bsnd(query, lens_q, "block_sparse_attention")
+        k4 = _tnd_as_bsnd(key, lens_kv, "block_sparse_attention")
+        v4 = _tnd_as_bsnd(value, lens_kv, "block_sparse_attention")
         layout = "BSND"
     else:
         q4, k4, v4, layout = query, key, value, "BNSD"
-        _check_lengths(actual_seq_lengths, query.shape[2], "block_sparse_attention")
-        _check_lengths(actual_seq_lengths_kv, key.shape[2], "block_sparse_attention")
-    want_lse = softmax_lse_flag != 0
+        full_q = lens_q is None or all(x == query.shape[2] for x in lens_q)
+        full_kv = lens_kv is None or all(x == key.shape[2] for x in lens_kv)
+        if not (full_q and full_kv):  # batch entries shorter than the tensor
+            res = _varlen("block_sparse_attention", query, key, value, block_sparse_mask, scale_value,
+                          lens_q if lens_q is not None else [query.shape[2]] * query.shape[0],
+                          lens_kv if lens_kv is not None else [key.shape[2]] * key.shape[0], "BNSD", return_lse=want_lse)
+            out, lse = res if want_lse else (res, None)
+            lse_out = lse.unsqueeze(-1) if want_lse else torch.empty(
+                (query.shape[0], query.shape[1], query.shape[2], 1), dtype=torch.float32, device=query.device)
+            return out, lse_out
     res = rf.block_sparse_attention_mask(q4, k4, v4, block_sparse_mask, scale_value, layout, return_lse=want_lse)
     out, lse = res if want_lse else (res, None)
     if q_input_layout == "TND":
@@ -147,10 +192,16 @@ def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blo
         raise RuntimeError(f"blockshape only supports [128, 128], got {list(blockshape)}")
     if attn_mask is not None or block_table is not None or mask_type != 0 or block_size != 0:
         raise RuntimeError("attn_mask / block_table / mask_type / block_size are not supported.")
-    if q_input_layout == "TND":
-        q4 = _tnd_as_bsnd(query, list(actual_seq_qlen) if actual_seq_qlen else None, "rainfusionattention")
-        k4 = _tnd_as_bsnd(key, list(actual_seq_kvlen) if actual_seq_kvlen else None, "rainfusionattention")
-        v4 = _tnd_as_bsnd(value, list(actual_seq_kvlen) if actual_seq_kvlen else None, "rainfusionattention")
+    lens_q = [int(x) for x in actual_seq_qlen] if actual_seq_qlen else None
+    lens_kv = [int(x) for x in actual_seq_kvlen] if actual_seq_kvlen else None
+    unequal = q_input_layout == "TND" and lens_q and lens_kv and (len(set(lens_q)) > 1 or len(set(lens_kv)) > 1)
+    if unequal:
+        q4 = k4 = v4 = None
+        layout, b, n = "TND", len(lens_q), query.shape[1]
+    elif q_input_layout == "TND":
+        q4 = _tnd_as_bsnd(query, lens_q, "rainfusionattention")
+        k4 = _tnd_as_bsnd(key, lens_kv, "rainfusionattention")
+        v4 = _tnd_as_bsnd(value, lens_kv, "rainfusionattention")
         layout = "BSND"
         b, n = q4.shape[0], q4.shape[2]
     else:
@@ -161,7 +212,7 @@ def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blo
     # The selection as an int8 mask: entry j of a row counts if j < select_num_idx and the id names a key block
     # (ids outside [0, kv_blocks) and entries past the count are dropped, so a malformed list cannot make the
     # kernel read outside its tables).  The mask form runs the paired two-pass kernel.
-    skv = k4.shape[2] if layout == "BNSD" else k4.shape[1]
+    skv = max(lens_kv) if unequal else (k4.shape[2] if layout == "BNSD" else k4.shape[1])
     kb = (skv + 127) // 128
     sel = select_idx.permute(1, 0, 2).to(torch.int64)                               # [N, qb, width]
     num = select_num_idx.permute(1, 0).to(torch.int64).unsqueeze(-1)                # [N, qb, 1]
@@ -170,6 +221,11 @@ def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blo
     mask = torch.zeros((n, sel.shape[1], kb + 1), dtype=torch.int8, device=sel.device)
     mask.scatter_(2, torch.where(valid, sel + 1, torch.zeros_like(sel)), 1)         # column 0 takes the dropped ones
     mask = mask[:, :, 1:].unsqueeze(0).expand(b, -1, -1, -1).contiguous()
+    if unequal:  # packed sequences of different lengths, the same selection for each
+        out, lse = _varlen("rainfusionattention", query, key, value, mask, scale, lens_q, lens_kv, "TND", return_lse=True)
+        lse_out = torch.zeros(query.shape, dtype=query.dtype, device=query.device)
+        lse_out[:, :, 0] = lse.to(query.dtype)
+        return out, lse_out
     out, lse = rf.block_sparse_attention_mask(q4, k4, v4, mask, scale, layout, return_lse=True)
     if q_input_layout == "TND":
         out = out.reshape(query.shape)
@@ -291,3 +347,65 @@ def ada_block_sparse_attention(query, key, value, sparse_mask, sparse_count_tabl
         num_key_value_heads=1 if num_key_value_heads is None else num_key_value_heads, scale_value=scale_value,
         causal=causal, inner_precise=inner_precise, pre_tokens=pre_tokens, next_tokens=next_tokens,
         actual_seq_lengths=actual_seq_lengths, actual_seq_lengths_kv=actual_seq_lengths_kv)
+
+
+# ---- FP8 / MXFP8 / RainFusion mask as ops --------------------------------------------------------------------------
+@register_ops.register_device_impl("fa_block_quant")
+def _fa_block_quant_impl(x, block_size=128, input_layout="BNSD"):
+    """-> (float8_e4m3fn [B, N, S, D], fp32 scale [B, N, ceil(S / block_size), 1]); see fa_block_quant_preprocess."""
+    from .quant.block_quant import fa_block_quant_preprocess
+    return fa_block_quant_preprocess(x, block_size=block_size, layout=input_layout)
+
+
+@register_ops.register_mindie_fake_op("fa_block_quant")
+def _fa_block_quant_fake(x, block_size=128, input_layout="BNSD"):
+    b, n, s = (x.shape[0], x.shape[1], x.shape[2]) if input_layout == "BNSD" else (x.shape[0], x.shape[2], x.shape[1])
+    return (torch.empty((b, n, s, x.shape[3]), device=x.device, dtype=torch.float8_e4m3fn),
+            torch.empty((b, n, (s + block_size - 1) // block_size, 1), device=x.device, dtype=torch.float32))
+
+
+@register_ops.register_device_impl("fp8_attention_fwd")
+def _fp8_attention_fwd_impl(query, key, value, scale_value=1.0, input_layout="BNSD", q_rot=None, k_rot=None,
+                            recipe="amax"):
+    from .quant.fp8_attention import fp8_attention_forward
+    return fp8_attention_forward(query, key, value, scale_value, input_layout, q_rot, k_rot, recipe)
+
+
+@register_ops.register_mindie_fake_op("fp8_attention_fwd")
+def _fp8_attention_fwd_fake(query, key, value, scale_value=1.0, input_layout="BNSD", q_rot=None, k_rot=None,
+                            recipe="amax"):
+    return torch.empty_like(query)
+
+
+@register_ops.register_device_impl("mxfp8_gemm_swiglu")
+def _mxfp8_gemm_swiglu_impl(x, weight, weight_scale, bias=None, swiglu=True):
+    """x [.., K] bf16/fp16 (quantised here, per 32 values along K), weight E4M3 [Nw, K] with E8M0 scales
+    [Nw, K/32]; ``swiglu``: weight rows are [gate | up] and the result is silu(gate) * up [.., Nw/2]."""
+    from .quant.mxfp8 import mx_quantize, mxfp8_matmul
+    x2 = x.reshape(-1, x.shape[-1])
+    xq, xs = mx_quantize(x2)
+    out = mxfp8_matmul(xq, xs, weight, weight_scale, bias, x.dtype, swiglu)
+    return out.view(*x.shape[:-1], out.shape[-1])
+
+
+@register_ops.register_mindie_fake_op("mxfp8_gemm_swiglu")
+def _mxfp8_gemm_swiglu_fake(x, weight, weight_scale, bias=None, swiglu=True):
+    nout = weight.shape[0] // 2 if swiglu else weight.shape[0]
+    return torch.empty((*x.shape[:-1], nout), device=x.device, dtype=x.dtype)
+
+
+@register_ops.register_device_impl("rf_block_mask")
+def _rf_block_mask_impl(qkv_pool, txt_len, sparsity, scale, latent_shape, input_layout="BNSD",
+                        protect_first_frame=True, keep_diagonal=False):
+    from .flash_attn.rainfusion import get_blockwise_mask
+    return get_blockwise_mask(qkv_pool, txt_len, sparsity, scale, 128, list(latent_shape), list(latent_shape),
+                              input_layout, return_binary=True, protect_first_frame=protect_first_frame,
+                              keep_diagonal=keep_diagonal)
+
+
+@register_ops.register_mindie_fake_op("rf_block_mask")
+def _rf_block_mask_fake(qkv_pool, txt_len, sparsity, scale, latent_shape, input_layout="BNSD",
+                        protect_first_frame=True, keep_diagonal=False):
+    b = qkv_pool.shape[0] // 3
+    n, nb = (qkv_pool.shape[1], qkv_pool.shape[2]) if input_layout == "BNSD" else (qkv_pool.shape[2], qkv_pool.shape[1])
+    return torch.empty((b, n, nb, nb), device=qkv_pool.device, dtype=torch.int8)

@@ -84,7 +84,7 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
                     mask = mask.contiguous()
                 m_sb = mask.stride(0) if mask.shape[0] > 1 else 0
                 m_sn = mask.stride(1) if mask.shape[1] > 1 else 0
-                m_sq = mask.stride(2) if sq > 1 else skv
+                m_sq = mask.stride(2) if sq > 1 else skv  # 0 for a mask expanded over the queries
             rc = _native.lib().mindiesd_flash_attention_general_fwd(
                 query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if lse is not None else None, _native.DTYPE_CODE[query.dtype],
@@ -94,31 +94,62 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
     return (out, lse) if return_lse else out
 
 
-def flash_attention_varlen(q, k, v, seqlens_q, seqlens_k, scale, causal=False):
-    """Packed sequences: q [Tq, N, D], k / v [Tk, Nkv, D]; sequence i owns ``seqlens_q[i]`` query tokens and
-    ``seqlens_k[i]`` key tokens, stored back to back.  Returns [Tq, N, D]."""
-    _check_qkv(q, k, v)
-    if q.dim() != 3 or k.shape != v.shape or k.dim() != 3 or q.shape[1] % k.shape[1] != 0:
-        raise ParametersInvalid("Inconsistent query/key/value shapes.")
+def _varlen_meta(cu_q, cu_k, total_q, total_k, device):
+    """Cumulative lengths -> (int32 [B, 4] device table {first query token, query count, first key token, key
+    count}, longest query count, longest key count, B).  Host lists / CPU tensors are validated and give exact
+    bounds; device tensors are turned into the table on the device without a host synchronisation - the bounds
+    are then the token totals (workgroups past a sequence's end return at once) and the entries are clamped to the
+    tensors instead of validated."""
+    on_device = isinstance(cu_q, torch.Tensor) and cu_q.is_cuda and isinstance(cu_k, torch.Tensor) and cu_k.is_cuda
+    if on_device:
+        if cu_q.dim() != 1 or cu_k.dim() != 1 or cu_q.shape[0] != cu_k.shape[0] or cu_q.shape[0] < 2:
+            raise ParametersInvalid("cu_seqlens_q and cu_seqlens_k must be 1-D with batch_size + 1 entries each.")
+        cq, ck = cu_q.to(device=device, dtype=torch.int64), cu_k.to(device=device, dtype=torch.int64)
+        sq0, sk0 = cq[:-1].clamp(0, total_q), ck[:-1].clamp(0, total_k)
+        lq = (cq[1:] - cq[:-1]).clamp(min=0)
+        lk = (ck[1:] - ck[:-1]).clamp(min=0)
+        lq, lk = torch.minimum(lq, total_q - sq0), torch.minimum(lk, total_k - sk0)
+        meta = torch.stack([sq0, lq, sk0, lk], dim=1).to(torch.int32).contiguous()
+        return meta, total_q, max(total_k, 1), cq.shape[0] - 1
+    def lengths(cu, name):
+        vals = [int(x) for x in (cu.detach().cpu().tolist() if isinstance(cu, torch.Tensor) else cu)]
+        if len(vals) < 2 or vals[0] != 0 or any(b < a for a, b in zip(vals, vals[1:])):
+            raise ParametersInvalid(f"{name} must start at 0, be non-decreasing and hold batch_size + 1 entries, "
+                                    f"but got {vals}.")
+        return [b - a for a, b in zip(vals, vals[1:])]
+    seqlens_q, seqlens_k = lengths(cu_q, "cu_seqlens_q"), lengths(cu_k, "cu_seqlens_k")
     if len(seqlens_q) != len(seqlens_k) or len(seqlens_q) == 0:
         raise ParametersInvalid("cu_seqlens_q and cu_seqlens_k must describe the same, non-zero number of sequences.")
-    if min(seqlens_q) < 0 or min(seqlens_k) < 0 or sum(seqlens_q) != q.shape[0] or sum(seqlens_k) != k.shape[0]:
+    if sum(seqlens_q) != total_q or sum(seqlens_k) != total_k:
         raise ParametersInvalid("The cumulative sequence lengths do not match the token dimensions of q / k.")
-    q, k, v = _aligned(q), _aligned(k), _aligned(v)
-    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     meta, oq, ok = [], 0, 0
     for lq, lk in zip(seqlens_q, seqlens_k):
         meta += [oq, lq, ok, lk]
         oq += lq
         ok += lk
-    if max(seqlens_q) == 0:
+    meta_t = torch.tensor(meta, dtype=torch.int32).view(-1, 4).to(device, non_blocking=True)
+    return meta_t, max(seqlens_q), max(max(seqlens_k), 1), len(seqlens_q)
+
+
+def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=False):
+    """Packed sequences: q [Tq, N, D], k / v [Tk, Nkv, D]; ``cu_seqlens_q`` / ``cu_seqlens_k``: cumulative sequence
+    lengths (batch + 1 entries; lists, CPU tensors or device tensors - the latter are used without a host
+    synchronisation).  Returns [Tq, N, D]."""
+    _check_qkv(q, k, v)
+    if q.dim() != 3 or k.shape != v.shape or k.dim() != 3 or q.shape[1] % k.shape[1] != 0:
+        raise ParametersInvalid("Inconsistent query/key/value shapes.")
+    q, k, v = _aligned(q), _aligned(k), _aligned(v)
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if q.shape[0] == 0:
         return out
-    meta_t = torch.tensor(meta, dtype=torch.int32).to(q.device, non_blocking=True)
+    meta_t, max_q, max_k, nseq = _varlen_meta(cu_seqlens_q, cu_seqlens_k, q.shape[0], k.shape[0], q.device)
+    if max_q == 0:
+        return out
     tn = lambda t: (0, t.stride(1), t.stride(0))  # (batch, head, token) strides of a [T, N, D] tensor
     with torch.cuda.device(q.device):
         rc = _native.lib().mindiesd_flash_attention_general_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None, _native.DTYPE_CODE[q.dtype],
-            len(seqlens_q), q.shape[1], k.shape[1], max(seqlens_q), max(max(seqlens_k), 1), q.shape[2],
+            nseq, q.shape[1], k.shape[1], max_q, max_k, q.shape[2],
             *tn(q), *tn(k), *tn(v), *tn(out), float(scale), meta_t.data_ptr(), int(bool(causal)), None, 0, 0, 0,
             _native.stream_ptr(q.device))
     _native.check(rc, "mindiesd_flash_attention_general_fwd")

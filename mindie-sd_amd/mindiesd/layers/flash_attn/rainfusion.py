@@ -271,6 +271,9 @@ def token_order(latent_shape, txt_len, device):
         with torch.cuda.device(dev):
             rc = _native.lib().mindiesd_rf_token_order(tok.data_ptr(), s, t, h, w, int(txt_len), _native.stream_ptr(dev))
         _native.check(rc, "mindiesd_rf_token_order")
+        # the table is reused by later calls on whatever stream is current then: wait once, here, for the kernel
+        # that fills it
+        torch.cuda.current_stream(dev).synchronize()
         if len(_token_order_cache) >= 16:
             _token_order_cache.clear()
         _token_order_cache[key] = tok
@@ -364,6 +367,62 @@ def block_sparse_attention_mask(query, key, value, block_sparse_mask, scale, lay
         idx, cnt = mask_to_lists(m8)
         return block_sparse_attention_lists(q, k, v, idx, cnt, scale, layout, return_lse, order)
     _native.check(rc, "mindiesd_block_sparse_attention_paired_fwd")
+    return (out, lse) if return_lse else out
+
+
+def block_sparse_attention_varlen(query, key, value, block_sparse_mask, scale, seq_lens_q, seq_lens_kv, layout,
+                                  return_lse=False):
+    """Block-sparse attention with one length per batch entry (``actual_seq_lengths`` / ``actual_seq_lengths_kv`` of
+    the reference op, csrc/plugin/block_sparse_attention.cpp:42-66).
+    ``layout`` 'BNSD': query [B, N, S, D], sequence b uses its first ``seq_lens_q[b]`` query and ``seq_lens_kv[b]``
+    key tokens; the other output rows are zero.  'TND': packed [T, N, D] tensors, sequence b follows sequence b - 1.
+    ``block_sparse_mask`` [B, N, ceil(max q len / 128), ceil(max kv len / 128)].  Returns the output like ``query``
+    (and the log-sum-exp [B, N, S] / [T, N] with ``return_lse``)."""
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype not in _native.DTYPE_CODE or t.shape[-1] != HEAD_DIM:
+            raise ParametersInvalid(f"{name} must be a bf16/fp16 GPU tensor with head_dim {HEAD_DIM}.")
+    q, k, v = _aligned(query), _aligned(key), _aligned(value)
+    lq, lk = [int(x) for x in seq_lens_q], [int(x) for x in seq_lens_kv]
+    b = len(lq)
+    if b == 0 or len(lk) != b or min(lq) <= 0 or min(lk) <= 0:
+        raise ParametersInvalid("sequence lengths must be positive, one per batch entry for queries and for keys.")
+    if layout == "TND":
+        if q.dim() != 3 or k.dim() != 3 or sum(lq) != q.shape[0] or sum(lk) != k.shape[0] or k.shape != v.shape:
+            raise ParametersInvalid("TND layout: [T, N, D] tensors whose token counts equal the sums of the lengths.")
+        n, nkv = q.shape[1], k.shape[1]
+        q_str, k_str, v_str = (0, q.stride(1), q.stride(0)), (0, k.stride(1), k.stride(0)), (0, v.stride(1), v.stride(0))
+        starts_q = [sum(lq[:i]) for i in range(b)]
+        starts_k = [sum(lk[:i]) for i in range(b)]
+        out = torch.empty_like(q)
+        lse = torch.empty((q.shape[0], n), dtype=torch.float32, device=q.device) if return_lse else None
+    elif layout == "BNSD":
+        if q.dim() != 4 or k.dim() != 4 or q.shape[0] != b or k.shape[0] != b or k.shape != v.shape:
+            raise ParametersInvalid("BNSD layout: 4-D tensors with one length per batch entry.")
+        if max(lq) > q.shape[2] or max(lk) > k.shape[2]:
+            raise ParametersInvalid("a sequence length exceeds the tensor.")
+        n, nkv = q.shape[1], k.shape[1]
+        q_str, k_str, v_str = _strides_bns(q, layout), _strides_bns(k, layout), _strides_bns(v, layout)
+        starts_q = starts_k = [0] * b
+        out = torch.zeros_like(q)
+        lse = torch.zeros((b, n, q.shape[2]), dtype=torch.float32, device=q.device) if return_lse else None
+    else:
+        raise ParametersInvalid(f"layout must be 'BNSD' or 'TND', but got {layout}.")
+    if n % nkv != 0 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ParametersInvalid("Inconsistent query/key/value head counts or dtypes.")
+    sq, skv = max(lq), max(lk)
+    qb, kb = (sq + BLOCK - 1) // BLOCK, (skv + BLOCK - 1) // BLOCK
+    if block_sparse_mask.dim() != 4 or tuple(block_sparse_mask.shape) != (b, n, qb, kb):
+        raise ParametersInvalid(f"block_sparse_mask must be [B, N, {qb}, {kb}], but got {tuple(block_sparse_mask.shape)}.")
+    idx, cnt = mask_to_lists(block_sparse_mask)
+    meta = torch.tensor([[starts_q[i], lq[i], starts_k[i], lk[i]] for i in range(b)], dtype=torch.int32).to(q.device)
+    o_str = (0, out.stride(1), out.stride(0)) if layout == "TND" else _strides_bns(out, layout)
+    with torch.cuda.device(q.device):
+        rc = _native.lib().mindiesd_block_sparse_attention_general_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
+            _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1], *q_str, *k_str, *v_str, *o_str, float(scale),
+            idx.data_ptr(), cnt.data_ptr(), idx.shape[3], meta.data_ptr(), int(layout == "TND"), 0,
+            _native.stream_ptr(q.device))
+    _native.check(rc, "mindiesd_block_sparse_attention_general_fwd")
     return (out, lse) if return_lse else out
 
 

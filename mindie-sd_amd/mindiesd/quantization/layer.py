@@ -4,15 +4,15 @@ from torch import nn
 
 from ..layers.quant.fp8_attention import fp8_attention_forward
 from ..layers.quant.mxfp8 import mx_quantize, mxfp8_matmul
+from ..utils.exception import ParametersInvalid
 
 
 def _get_weight(weights, name):
-    """``weights`` is a mapping name -> tensor (the reference reads the same names from a
-    safetensors handle, mindiesd/quantization/quantize.py:229-238)."""
-    if weights is None:
-        raise ValueError(f"weights mapping is required to build a quantised layer (missing '{name}')")
-    w = weights.get_tensor(name) if hasattr(weights, "get_tensor") else weights[name]
-    return w
+    """``weights`` is a safetensors handle (``keys()`` / ``get_tensor``; mindiesd/quantization/quantize.py:229-238) or a
+    plain mapping name -> tensor; a missing entry raises ParametersInvalid (quantization/utils.py:70-87)."""
+    if weights is None or name not in weights.keys():
+        raise ParametersInvalid(f"Critical parameter missing: {name}.")
+    return weights.get_tensor(name) if hasattr(weights, "get_tensor") else weights[name]
 
 
 class FP8RotateQuantFA(nn.Module):

@@ -156,6 +156,28 @@ def test_op_schemas_and_fake_impls():
         assert piece in schema, (piece, schema)
 
 
+def test_new_ops_have_schemas_and_fake_impls():
+    """The FP8 / MXFP8 / RainFusion-mask ops of this build on meta tensors (what torch.compile sees)."""
+    import mindiesd  # noqa: F401
+    x = torch.empty(2, 300, 4, 128, device="meta", dtype=torch.bfloat16)
+    codes, scale = torch.ops.mindiesd.fa_block_quant(x, block_size=256, input_layout="BSND")
+    assert codes.shape == (2, 4, 300, 128) and codes.dtype == torch.float8_e4m3fn
+    assert scale.shape == (2, 4, 2, 1) and scale.dtype == torch.float32
+    rot = torch.empty(128, 128, device="meta", dtype=torch.bfloat16)
+    out = torch.ops.mindiesd.fp8_attention_fwd(x, x, x, scale_value=0.1, input_layout="BSND", q_rot=rot, k_rot=rot)
+    assert out.shape == x.shape and out.dtype == x.dtype
+    a = torch.empty(3, 50, 256, device="meta", dtype=torch.float16)
+    w = torch.empty(512, 256, device="meta", dtype=torch.float8_e4m3fn)
+    ws = torch.empty(512, 8, device="meta", dtype=torch.uint8)
+    assert torch.ops.mindiesd.mxfp8_gemm_swiglu(a, w, ws).shape == (3, 50, 256)
+    assert torch.ops.mindiesd.mxfp8_gemm_swiglu(a, w, ws, swiglu=False).shape == (3, 50, 512)
+    pool = torch.empty(3, 4, 9, 128, device="meta", dtype=torch.bfloat16)
+    mask = torch.ops.mindiesd.rf_block_mask(pool, 0, 0.5, 0.09, [2, 24, 24])
+    assert mask.shape == (1, 4, 9, 9) and mask.dtype == torch.int8
+    for name in ("fa_block_quant", "fp8_attention_fwd", "mxfp8_gemm_swiglu", "rf_block_mask"):
+        assert hasattr(torch.ops.mindiesd, name)
+
+
 def test_sparse_front_door_checks():
     import mindiesd
     q = torch.randn(1, 2, 256, 128, dtype=torch.bfloat16)

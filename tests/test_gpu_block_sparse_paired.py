@@ -160,3 +160,43 @@ def test_rainfusionattention_lists_with_malformed_entries(cuda):
     want, _ = torch.ops.mindiesd.block_sparse_attention(q, k, v, keep.to(cuda), scale_value=128 ** -0.5)
     assert torch.equal(out, want)
     assert oa.ref_compare(oa.block_sparse_attention(q.cpu(), k.cpu(), v.cpu(), keep.numpy()), out.cpu(), 2.0 ** -6)[1]
+
+
+def test_block_sparse_op_with_per_batch_lengths(cuda):
+    """actual_seq_lengths / actual_seq_lengths_kv of the block_sparse_attention op
+    (csrc/plugin/block_sparse_attention.cpp:42-66): batch entries shorter than the BNSD tensor, and TND tensors packing
+    sequences of different lengths; each sequence against the oracle on its own slice."""
+    import mindiesd  # noqa: F401
+    n, s = 2, 900
+    lens_q, lens_kv = [900, 333], [700, 900]
+    q, k, v = _rand((2, n, s, 128), 31), _rand((2, n, s, 128), 32), _rand((2, n, s, 128), 33)
+    nb = (s + 127) // 128
+    m = _banded_mask(2, n, nb, nb, seed=34, period=3, keep=0.5)
+    m[:, :, 3] = m[:, :, 2]
+    out, lse = torch.ops.mindiesd.block_sparse_attention(
+        q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda), scale_value=128 ** -0.5,
+        actual_seq_lengths=lens_q, actual_seq_lengths_kv=lens_kv, softmax_lse_flag=1)
+    assert out.shape == q.shape and lse.shape == (2, n, s, 1)
+    for b in range(2):
+        lq, lk = lens_q[b], lens_kv[b]
+        qb, kb = (lq + 127) // 128, (lk + 127) // 128
+        want = oa.block_sparse_attention(q[b:b + 1, :, :lq], k[b:b + 1, :, :lk], v[b:b + 1, :, :lk], m[b:b + 1, :, :qb, :kb].numpy())
+        assert oa.ref_compare(want, out[b:b + 1, :, :lq].cpu(), 2.0 ** -6)[1]
+        assert not out[b, :, lq:].any()
+    # the same two sequences packed as TND
+    qt = torch.cat([q[b, :, :lens_q[b]].transpose(0, 1) for b in range(2)]).contiguous()
+    kt = torch.cat([k[b, :, :lens_kv[b]].transpose(0, 1) for b in range(2)]).contiguous()
+    vt = torch.cat([v[b, :, :lens_kv[b]].transpose(0, 1) for b in range(2)]).contiguous()
+    out_t, lse_t = torch.ops.mindiesd.block_sparse_attention(
+        qt.to(cuda), kt.to(cuda), vt.to(cuda), m.to(torch.int8).to(cuda), q_input_layout="TND", kv_input_layout="TND",
+        scale_value=128 ** -0.5, actual_seq_lengths=lens_q, actual_seq_lengths_kv=lens_kv, softmax_lse_flag=1)
+    assert out_t.shape == qt.shape and lse_t.shape == (sum(lens_q), n, 1)
+    t0 = 0
+    for b in range(2):
+        lq = lens_q[b]
+        assert torch.equal(out_t[t0:t0 + lq].transpose(0, 1), out[b, :, :lq])
+        assert torch.equal(lse_t[t0:t0 + lq, :, 0].transpose(0, 1), lse[b, :, :lq, 0])
+        t0 += lq
+    with pytest.raises(RuntimeError):
+        torch.ops.mindiesd.block_sparse_attention(q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda),
+                                                  actual_seq_lengths=[901, 5], actual_seq_lengths_kv=lens_kv)

@@ -158,3 +158,33 @@ def test_fp8_rotate_quant_fa_module(cuda):
     assert out.shape == q.shape and cosine(out, ref) > 0.995
     with pytest.raises(ValueError):
         mod(q.to(cuda), k.to(cuda), v.to(cuda), layout="SBH")
+
+
+def test_ops_match_the_python_functions_and_trace(cuda):
+    """torch.ops.mindiesd.{fa_block_quant, fp8_attention_fwd, mxfp8_gemm_swiglu, rf_block_mask} give what the Python
+    entry points give, and a function built from them compiles as one graph (fake implementations present)."""
+    import mindiesd  # noqa: F401
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    from mindiesd.layers.quant import fa_block_quant_preprocess, fp8_attention_forward, mx_quantize, mxfp8_matmul
+    q, k, v = (t.to(cuda) for t in _outlier_inputs((1, 2, 700, 128), seed=11))
+    codes, scale = torch.ops.mindiesd.fa_block_quant(q, 128, "BNSD")
+    c2, s2 = fa_block_quant_preprocess(q, block_size=128)
+    assert torch.equal(codes.view(torch.uint8), c2.view(torch.uint8)) and torch.equal(scale, s2)
+    out = torch.ops.mindiesd.fp8_attention_fwd(q, k, v, 128 ** -0.5)
+    assert torch.equal(out, fp8_attention_forward(q, k, v))
+    x = torch.randn(5, 30, 256, device=cuda).to(torch.bfloat16)
+    wq, ws = mx_quantize((torch.randn(512, 256, device=cuda) * 0.05).to(torch.bfloat16))
+    y = torch.ops.mindiesd.mxfp8_gemm_swiglu(x, wq, ws)
+    xq, xs = mx_quantize(x.reshape(-1, 256))
+    assert torch.equal(y, mxfp8_matmul(xq, xs, wq, ws, None, torch.bfloat16, True).view(5, 30, 256))
+    grid = (2, 24, 24)
+    qq, kk, vv = (torch.randn(1, 2, 2 * 24 * 24, 128, device=cuda).to(torch.bfloat16) for _ in range(3))
+    _, _, _, pool = rf.do_tensor_rearrange_pooling(qq, kk, vv, 0, 128, grid, grid, "BNSD")
+    m = torch.ops.mindiesd.rf_block_mask(pool, 0, 0.6, 128 ** -0.5, list(grid))
+    assert torch.equal(m, rf.get_blockwise_mask(pool, 0, 0.6, 128 ** -0.5, 128, grid, grid, "BNSD", return_binary=True))
+
+    def fn(a, b, c, xx):
+        return torch.ops.mindiesd.fp8_attention_fwd(a, b, c, 128 ** -0.5), torch.ops.mindiesd.mxfp8_gemm_swiglu(xx, wq, ws)
+
+    o1, o2 = torch.compile(fn, backend="eager", fullgraph=True)(q, k, v, x)
+    assert torch.equal(o1, out) and torch.equal(o2, y)

@@ -116,3 +116,19 @@ def test_varlen_and_mask_errors(cuda):
         mindiesd.attention_forward(x, x, x, attn_mask=torch.ones(3, 64, 64, dtype=torch.bool, device=cuda))
     with pytest.raises(ParametersInvalid, match="attn_mask"):
         mindiesd.attention_forward(x, x, x, attn_mask=torch.ones(63, 64, dtype=torch.bool, device=cuda))
+
+
+def test_key_padding_mask_expanded_over_queries(cuda):
+    """[B, 1, 1, Skv] key-padding mask expanded to [B, 1, Sq, Skv]: a view whose query stride is 0 runs without
+    being materialised."""
+    import mindiesd
+    b, n, sq, skv = 2, 2, 260, 333
+    q, k, v = _rand((b, n, sq, 128), 21), _rand((b, n, skv, 128), 22), _rand((b, n, skv, 128), 23)
+    keep = torch.ones(b, 1, 1, skv, dtype=torch.bool)
+    keep[0, ..., 300:] = False
+    keep[1, ..., 17:40] = False
+    ref = attention_math(q, k, v, keep.expand(b, n, sq, skv), head_first=True)
+    view = keep.to(cuda).expand(b, 1, sq, skv)
+    assert view.stride(2) == 0
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=view, head_first=True).cpu()
+    _check(out, ref)

@@ -73,3 +73,42 @@ def test_gemm_errors(cuda):
         mxfp8_matmul(xq, xs, xq, xs)            # K not a multiple of 128
     with pytest.raises(ParametersInvalid):
         mx_quantize(_rand((4, 40), 8).to(cuda))  # K not a multiple of 32
+
+
+def test_quantize_injected_layers_match_direct_calls(cuda, tmp_path):
+    """quantize() on a toy block (descriptor + safetensors written here): the swapped-in linear equals the direct
+    MXFP8 GEMM on the same tensors, the attached fa_quant equals the direct FP8 attention call."""
+    import json
+    import os
+    from safetensors.torch import save_file
+    from torch import nn
+    from mindiesd import quantize
+    from mindiesd.layers.quant import fp8_attention_forward, mx_quantize, mxfp8_matmul
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = nn.Linear(256, 512)
+            self.attn = nn.Identity()
+
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(512, 256, generator=g) * 0.05).to(torch.bfloat16).to(cuda)
+    wq, ws = mx_quantize(w)
+    bias = torch.randn(512, generator=g)
+    rot = torch.linalg.qr(torch.randn(128, 128, generator=g))[0].to(torch.bfloat16).contiguous()
+    weights = {"up.weight": wq.cpu(), "up.weight_scale": ws.view(torch.uint8).cpu().reshape(512, -1, 2).contiguous(),
+               "up.bias": bias, "attn.q_rot": rot, "attn.k_rot": rot.clone()}
+    des = {"model_quant_type": "W8A8_MXFP8", "up.weight": "W8A8_MXFP8", "attn.fa_q.scale": "FP8_DYNAMIC"}
+    with open(os.path.join(tmp_path, "d.json"), "w") as f:
+        json.dump(des, f)
+    save_file(weights, os.path.join(tmp_path, "quant_model_weight_w8a8_mxfp8.safetensors"))
+    model = quantize(Block(), os.path.join(str(tmp_path), "d.json")).to(cuda)
+    x = torch.randn(3, 40, 256, generator=g).to(torch.bfloat16).to(cuda)
+    got = model.up(x)
+    xq, xs = mx_quantize(x.reshape(-1, 256))
+    want = mxfp8_matmul(xq, xs, wq, ws, bias.to(cuda), torch.bfloat16, False).view(3, 40, 512)
+    assert got.shape == (3, 40, 512) and torch.equal(got, want)
+    q, k, v = (torch.randn(1, 2, 300, 128, generator=g).to(torch.bfloat16).to(cuda) for _ in range(3))
+    a = model.attn.fa_quant(q, k, v, layout="BNSD")
+    b = fp8_attention_forward(q, k, v, layout="BNSD", q_rot=rot.to(cuda), k_rot=rot.to(cuda))
+    assert torch.equal(a, b)
