@@ -113,12 +113,17 @@ def per_channel_quant(v):
     return torch.from_numpy(e4m3_encode(vf / sc[..., None, :])), torch.from_numpy(sc)
 
 
-def fp8_attention(query, key, value, scale=None, pow2=False):
+def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False):
     """FP8 attention of the Wan2.1-14B 480p workload, BNSD: Q and K quantised per (head, 128-token
-    block) over all channels, V per (head, channel); everything is dequantised and run through plain
-    softmax(scale QK^T)V in fp32; bf16-typed output.  (The quantise -> dequantise path: the GPU kernel
-    additionally re-quantises the probabilities per tile, which this oracle does not model; the
-    stated tolerance, cosine >= 0.999, covers it.)"""
+    block) over all channels, V per (head, channel); bf16-typed output.
+    ``requant_p=False``: the quantise -> dequantise path - everything is dequantised and run through plain
+    softmax(scale QK^T)V in fp32.
+    ``requant_p=True``: additionally the workload's "P re-quantised to e4m3 per tile", with the choices of the GPU
+    kernel: keys in tiles of 128; per tile P = 2^4 * exp2(score - reference) rounded to E4M3 (ties to even), where
+    the reference is a running maximum per query row that is only moved when, in the row's group of 32 consecutive
+    query rows, some row's tile maximum exceeds its reference by more than 2^4 (so P <= 256 < 448); the
+    denominator is the sum of the ROUNDED probabilities, the numerator their product with the V codes; both are
+    rescaled by 2^(old - new reference) when the reference moves."""
     d = query.shape[-1]
     if scale is None:
         scale = d ** -0.5
@@ -132,6 +137,8 @@ def fp8_attention(query, key, value, scale=None, pow2=False):
         qc, qs = dynamic_block_quant(query, 128, d)
         kc, ks = dynamic_block_quant(key, 128, d)
     vc, vs = per_channel_quant(value)
+    if requant_p:
+        return _fp8_attention_requant(qc, qs, kc, ks, vc, vs, np.float32(scale * 1.4426950408889634), pow2).to(query.dtype)
     qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, 128, d)
     vd = torch.from_numpy(e4m3_decode(vc.numpy())) * vs[..., None, :]
     out = torch.empty(query.shape, dtype=torch.float32)
@@ -139,6 +146,57 @@ def fp8_attention(query, key, value, scale=None, pow2=False):
         s = (qd[..., r0:r0 + 2048, :] @ kd.transpose(-1, -2)) * scale
         out[..., r0:r0 + 2048, :] = torch.softmax(s, dim=-1) @ vd
     return out.to(query.dtype)
+
+
+P_SHIFT, P_TAU, ROW_GROUP, KEY_TILE = np.float32(4.0), np.float32(4.0), 32, 128
+
+
+def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2):
+    """The tile loop behind ``fp8_attention(requant_p=True)`` on the quantised operands (codes + scales)."""
+    q8, k8, v8 = e4m3_decode(qc.numpy()), e4m3_decode(kc.numpy()), e4m3_decode(vc.numpy())
+    qsn, ksn, vsn = qs.numpy()[..., 0], ks.numpy()[..., 0], vs.numpy()
+    b, n, sq, d = q8.shape
+    skv = k8.shape[2]
+    out = np.zeros((b, n, sq, d), dtype=np.float32)
+    for bi in range(b):
+        for ni in range(n):
+            for r0 in range(0, sq, ROW_GROUP):
+                r1 = min(r0 + ROW_GROUP, sq)
+                rows = r1 - r0
+                qsc = qsn[bi, ni, r0 // 128]
+                m_run = np.full(rows, 0.0 if pow2 else -np.inf, dtype=np.float32)
+                l_run = np.zeros(rows, dtype=np.float32)
+                o_run = np.zeros((rows, d), dtype=np.float32)
+                first = True
+                for t0 in range(0, skv, KEY_TILE):
+                    t1 = min(t0 + KEY_TILE, skv)
+                    raw = q8[bi, ni, r0:r1] @ k8[bi, ni, t0:t1].T                     # exact sums of code products
+                    if pow2:  # the scales are powers of two (applied by the matrix instruction's exponents)
+                        s = (raw * (qsc * ksn[bi, ni, t0 // 128])).astype(np.float32)
+                        mx = s.max(axis=1) - m_run
+                        if first or (mx > P_TAU).any():
+                            delta = mx if first else np.maximum(mx, np.float32(0))
+                            alpha = np.exp2(-delta).astype(np.float32)
+                            m_run = m_run + delta
+                            l_run *= alpha
+                            o_run *= alpha[:, None]
+                    else:     # amax/448 scales folded into the softmax scale of the tile
+                        c = np.float32(np.float32(qsc * scale_log2) * ksn[bi, ni, t0 // 128])
+                        s = (raw * c).astype(np.float32)
+                        mx = s.max(axis=1)
+                        if (mx > m_run + P_TAU).any():
+                            m_new = np.maximum(m_run, mx)
+                            alpha = np.where(np.isinf(m_run), np.float32(0), np.exp2(m_run - m_new)).astype(np.float32)
+                            m_run = m_new
+                            l_run *= alpha
+                            o_run *= alpha[:, None]
+                    first = False
+                    p8 = e4m3_round(np.exp2(s - (m_run - P_SHIFT)[:, None]).astype(np.float32))
+                    l_run += p8.sum(axis=1, dtype=np.float32)
+                    o_run += p8 @ v8[bi, ni, t0:t1]
+                inv = np.where(l_run > 0, np.float32(1) / np.maximum(l_run, np.float32(1e-30)), np.float32(0))
+                out[bi, ni, r0:r1] = o_run * inv[:, None] * vsn[bi, ni][None, :]
+    return torch.from_numpy(out)
 
 
 # ---- MX (microscaling) ----------------------------------------------------------------------------------

@@ -110,6 +110,15 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
     assert cos >= 0.999, f"cosine {cos}"
     # coarse guard against gross outliers: E4M3 probabilities carry 2^-4 relative noise per element
     assert err.max() < 0.2 * want.float().abs().max()
+    # against the oracle that re-quantises P the way the kernel does (same tiles, same reference rule, same
+    # rounding): what is left is the summation order, the hardware's exp2 and a probability now and then landing on
+    # the neighbouring E4M3 number
+    mirror = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True)
+    cos_m = cosine(out, mirror)
+    err_m = (out.float() - mirror.float()).abs()
+    print(f"   vs the P-requantising oracle: cosine {cos_m:.7f}, max-abs {err_m.max():.5f}")
+    assert cos_m >= 0.99999, f"cosine {cos_m}"
+    assert err_m.max() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
 
 
 @pytest.mark.parametrize("layout,dtype", [("BNSD", torch.bfloat16), ("BSND", torch.bfloat16), ("BNSD", torch.float16)])

@@ -144,3 +144,30 @@ def test_fp8_attention_recipes_agree_with_each_other_and_with_plain_attention():
     a, b = oq.fp8_attention(q, k, v), oq.fp8_attention(q, k, v, pow2=True)
     ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=True)
     assert cosine(a, b) > 0.997 and cosine(b, ref) > 0.995 and cosine(a, ref) > 0.995
+
+
+@pytest.mark.parametrize("pow2", [False, True])
+def test_requantised_probabilities_stay_within_a_bound_of_the_plain_form(pow2):
+    """``fp8_attention(requant_p=True)`` (P rounded to E4M3 per 128-key tile, denominator from the rounded values,
+    lazily moved reference) against the plain quantise -> dequantise form: an E4M3 probability carries at most
+    2^-4 relative error, and the errors of a row average out over its keys - the outputs differ by far less than
+    2^-5 of the largest value, a factor on P that did not cancel or a missed rescale would not."""
+    import torch
+    g = torch.Generator().manual_seed(3)
+    def make():
+        x = torch.randn(1, 2, 700, 128, generator=g)
+        return torch.where(torch.rand(1, 2, 700, 128, generator=g) < 0.01, x * 8, x).to(torch.bfloat16)
+    q, k, v = make(), make(), make()
+    k[:, :, 300:] *= 1.5            # rising row maxima: the reference has to move after the first tile
+    a = oq.fp8_attention(q, k, v, pow2=pow2).float()
+    b = oq.fp8_attention(q, k, v, pow2=pow2, requant_p=True).float()
+    assert torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0) >= 0.9999
+    assert (a - b).abs().max() <= 2.0 ** -5 * v.float().abs().max()
+    # one key tile, uniform scores: every probability is the same power of two, the rounding is exact and the
+    # result is the mean of the (de)quantised values whatever the recipe does with the reference
+    kz = torch.zeros(1, 1, 100, 128, dtype=torch.bfloat16)
+    vz = make()[:, :1, :100]
+    out = oq.fp8_attention(q[:, :1, :40], kz, vz, pow2=pow2, requant_p=True).float()
+    codes, sc = oq.per_channel_quant(vz)
+    mean = (torch.from_numpy(oq.e4m3_decode(codes.numpy())) * sc[..., None, :]).mean(dim=-2, keepdim=True)
+    assert (out - mean.to(torch.bfloat16).float()).abs().max() <= 2.0 ** -7 * mean.abs().max()
