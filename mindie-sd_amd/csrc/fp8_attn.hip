@@ -401,7 +401,9 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   const float q_sc_raw = p.q_scale[(long long)bn * qblocks + qblk];
   const float q_sc = q_sc_raw * p.scale_log2;
   const int q_exp = (int)((__builtin_bit_cast(unsigned, q_sc_raw) >> 23) & 0xffu);  // E8M0 code of a power of two
-  const float* k_sc = p.k_scale + (long long)bn * kblocks;
+  // read through the constant address space: a scalar load, which does not queue behind the tile requests
+  typedef const __attribute__((address_space(4))) float* ConstF;
+  const ConstF k_sc = (ConstF)(uintptr_t)(p.k_scale + (long long)bn * kblocks);
 
   f32x16_t oacc[4];
 #pragma unroll
@@ -438,9 +440,17 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     }
   };
 
-  // operand read offsets: row = blk*32 + l32, bytes 64*ks + 32*h .. +32 = chunks 4*ks + 2*h, +1
+  // operand read addresses: row = blk*32 + l32, bytes 64*ks + 32*h .. +32 = chunks 4*ks + 2*h, +1 of the row.  The
+  // four per-lane addresses (k step x half of the 32 bytes) are kept in registers; stage, operand and 32-row block
+  // are compile-time constants that go into the offset field of the reads.
   const int row_off = l32 * 128;
   const int swz = (l32 >> 1) & 7;
+  unsigned rd[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      rd[ks][j] = (unsigned)(uintptr_t)smem + row_off + (((4 * ks + 2 * h + j) ^ swz) << 4);
 
   // Row sums come from the matrix core: one extra MFMA per 64 keys with an all-ones A operand
   // leaves sum_k P8[k][q] in every row of lacc, so the softmax needs no per-element additions and
@@ -451,45 +461,41 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   const i32x8_t ones8 = {0x38383838, 0x38383838, 0x38383838, 0x38383838,
                          0x38383838, 0x38383838, 0x38383838, 0x38383838};  // E4M3 1.0
 
+  // three stages: tile t + 2 is requested when tile t starts, so a request has two tile times to land
   if (n_tiles > 0) load_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);
+  if (n_tiles > 1) load_tile(1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0f74);  // all but the four requests of tile 1
   __syncthreads();
 
-  // The K scale of a tile is fetched one tile ahead and BEFORE that step's LDS-DMA requests: memory
-  // operations complete in order, so a scale requested after them could only be used once the whole next
-  // tile has landed, which would put that wait into the middle of every tile.
+  // The K scale of a tile is fetched one tile ahead.
   float k_sc_cur = n_tiles > 0 ? k_sc[0] : 0.f;
   auto tile_step = [&](const int t, auto stage_c) {
     constexpr int stage = decltype(stage_c)::value;
     const float k_sc_next = k_sc[t + 1 < n_tiles ? t + 1 : t];
-    // issued after the last tile as well (past the end of the buffers: reads as zeros, nobody uses it), so that
-    // the number of requests in flight behind the scale is the same on every path
-    load_tile(t + 1, stage ^ 1);
-    MSD_LDS const char* kb_base = smem + stage * kStage;
-    MSD_LDS const char* vb_base = kb_base + kTile;
+    // issued after the last tile as well (past the end of the buffers: nobody uses it), so that the number of
+    // requests in flight is the same on every path
+    load_tile(t + 2, (stage + 2) % 3);
 
     // ---- S^T = K Q^T (fp8, unscaled form of the scaled MFMA) ---------------------------------------------------
     f32x16_t sacc[4];
     const int k_exp = (int)((__builtin_bit_cast(unsigned, k_sc_cur) >> 23) & 0xffu);
-    if (!P2) {
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-    }
+    // the first product of a chain takes its seed as the C operand: kPShift - m (P2) or the constant zero (no
+    // accumulator is cleared by moves)
+    const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        MSD_LDS const char* src = kb_base + kb * 32 * 128 + row_off;
-        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h) ^ swz) << 4));
-        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(src + (((4 * ks + 2 * h + 1) ^ swz) << 4));
+        constexpr int kOff = stage * kStage;
+        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(uintptr_t)(rd[ks][0] + kOff + kb * 32 * 128);
+        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(uintptr_t)(rd[ks][1] + kOff + kb * 32 * 128);
         const i32x8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         if (P2)
           sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], ks == 0 ? negm : sacc[kb], 0, 0, 0,
                                                                      k_exp, 0, q_exp);
         else
-          sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
+          sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, qf[ks], ks == 0 ? zero16 : sacc[kb], 0, 0, 0, 0,
+                                                                     0, 0);
       }
     }
 
@@ -535,14 +541,6 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
           for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
       }
       first = false;
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4)
-          pf[kb >> 1][(kb & 1) * 4 + g4] =
-              pack4_e4m3_noclamp(fast_exp2(sacc[kb][4 * g4]), fast_exp2(sacc[kb][4 * g4 + 1]),
-                                 fast_exp2(sacc[kb][4 * g4 + 2]), fast_exp2(sacc[kb][4 * g4 + 3]));
-      }
     } else {
     mx *= c;
     if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau8) != 0) {
@@ -557,39 +555,68 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
     }
-    const float mc = (m_run == -INFINITY ? 0.f : m_run) - kPShift;
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4)
-        pf[kb >> 1][(kb & 1) * 4 + g4] = pack4_e4m3_noclamp(
-            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4], c, -mc)), fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 1], c, -mc)),
-            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 2], c, -mc)),
-            fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 3], c, -mc)));
-    }
     }  // !P2
-
-    // ---- O^T += V^T P^T (fp8), row sums ---------------------------------------------------------------------------
+    const float mc = P2 ? 0.f : (m_run == -INFINITY ? 0.f : m_run) - kPShift;
+    // probabilities of keys 64 * kk .. + 64 of the tile, rounded to E4M3 and packed as the B operand
+    auto exp_pack = [&](const int kk) {
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
+      for (int kb = 2 * kk; kb < 2 * kk + 2; ++kb) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          if (P2)
+            pf[kk][(kb & 1) * 4 + g4] =
+                pack4_e4m3_noclamp(fast_exp2(sacc[kb][4 * g4]), fast_exp2(sacc[kb][4 * g4 + 1]),
+                                   fast_exp2(sacc[kb][4 * g4 + 2]), fast_exp2(sacc[kb][4 * g4 + 3]));
+          else
+            pf[kk][(kb & 1) * 4 + g4] = pack4_e4m3_noclamp(fast_exp2(__builtin_fmaf(sacc[kb][4 * g4], c, -mc)),
+                                                           fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 1], c, -mc)),
+                                                           fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 2], c, -mc)),
+                                                           fast_exp2(__builtin_fmaf(sacc[kb][4 * g4 + 3], c, -mc)));
+        }
+      }
+    };
+    // ---- O^T += V^T P^T (fp8), row sums ---------------------------------------------------------------------------
+    auto pv = [&](const int kk) {
       lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones8, pf[kk], lacc, 0, 0, 0, 0, 0, 0);
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        MSD_LDS const char* src = vb_base + db * 32 * 128 + row_off;
-        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(src + (((4 * kk + 2 * h) ^ swz) << 4));
-        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(src + (((4 * kk + 2 * h + 1) ^ swz) << 4));
+        constexpr int kOff = stage * kStage + kTile;
+        const i32x4_t lo = *(MSD_LDS const i32x4_t*)(uintptr_t)(rd[kk][0] + kOff + db * 32 * 128);
+        const i32x4_t hi = *(MSD_LDS const i32x4_t*)(uintptr_t)(rd[kk][1] + kOff + db * 32 * 128);
         const i32x8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf[kk], oacc[db], 0, 0, 0, 0, 0, 0);
       }
+    };
+    // The products of the first 64 keys run on the matrix core while the vector unit rounds the probabilities of
+    // the other 64: the scheduler is told to put one product in front of every kValuPerMfma vector instructions.
+    exp_pack(0);
+    __builtin_amdgcn_sched_barrier(0);
+    pv(0);
+    exp_pack(1);
+    constexpr int kValuPerMfma = P2 ? 10 : 16;
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x402, kValuPerMfma, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    pv(1);
 
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
+    // tile t + 1 has to be there: everything but the four requests issued in this step
+    __builtin_amdgcn_s_waitcnt(0x0f74);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
   };
-  for (int t = 0; t < n_tiles; t += 2) {
+  for (int t = 0; t < n_tiles; t += 3) {
     tile_step(t, std::integral_constant<int, 0>{});
     if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
+    if (t + 2 < n_tiles) tile_step(t + 2, std::integral_constant<int, 2>{});
   }
+  // the requests past the last tile still write into the stages, which the output staging reuses
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
 
   // ---- epilogue: 1/l, per-channel V scale, transpose through LDS, coalesced store -----------------------------------
   // (the 2^kPShift factor is in both the accumulator and the running sum, so it cancels)
@@ -767,7 +794,7 @@ int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, 
   p.o = out; p.o_sb = o_sb; p.o_sn = o_sn; p.o_ss = o_ss;
   p.B = B; p.N = N; p.Sq = Sq; p.Skv = Skv; p.S128 = S128;
   p.scale_log2 = scale * 1.4426950408889634f;
-  constexpr int kLds = 8 * 32 * (256 + 8);  // output staging (66 KiB) > 2 stages x 32 KiB
+  constexpr int kLds = 3 * 32768;  // 3 stages x 32 KiB; the output staging (66 KiB) reuses them
   const int q_tiles = (Sq + 255) / 256;
   const int total = B * N * q_tiles;
   const int grid = (total + 7) / 8 * 8;
