@@ -100,6 +100,61 @@ def cpu_baseline_dense(cfg, target_s=12.0):
     }
 
 
+def cpu_baseline_sparse(cfg, device, target_s=8.0):
+    """The oracle's RainFusion pipeline on ONE head of the 14B 720p workload: window permutation + block means +
+    mask for the whole head, then the block-sparse attention of the first query blocks until about ``target_s``
+    seconds are spent; dense-equivalent TFLOP/s over the attended rows (permutation and mask time included
+    pro rata)."""
+    import torch
+    from oracle import rainfusion as orf
+    from oracle.attention import block_sparse_attention
+    one = dict(cfg, N=1)
+    q, k, v = (t.cpu() for t in smooth_field_inputs(one, device, seed=3))
+    s, d, grid = cfg["S"], cfg["D"], cfg["grid"]
+    t0 = time.perf_counter()
+    q_, k_, v_, pool = orf.do_tensor_rearrange_pooling(q, k, v, 0, 128, grid, grid, "BNSD")
+    mask = orf.get_blockwise_mask(pool, 0, 0.75, d ** -0.5, 128, grid, grid, "BNSD", return_binary=True,
+                                  keep_diagonal=True)
+    prep = time.perf_counter() - t0
+    nb = mask.shape[-2]
+    blocks, t1 = 0, time.perf_counter()
+    while blocks < nb and time.perf_counter() - t1 < target_s:
+        r = min(8, nb - blocks)
+        block_sparse_attention(q_[:, :, blocks * 128:(blocks + r) * 128], k_, v_, mask[:, :, blocks:blocks + r],
+                               scale=d ** -0.5)
+        blocks += r
+    att = time.perf_counter() - t1
+    rows = min(blocks * 128, s)
+    dt = att + prep * rows / s
+    return {"value": 4.0 * rows * s * d / dt / 1e12, "unit": "TFLOP/s (dense-equivalent)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle rf_v3 pipeline, one head of 40: permutation + block means + mask of the whole head "
+                      f"({prep:.1f} s, charged pro rata) and block-sparse attention of the first {blocks} of {nb} "
+                      f"query blocks ({att:.1f} s), mask density {float(mask.float().mean()):.3f}"}
+
+
+def cpu_baseline_gemm(target_s=8.0):
+    """The oracle's MXFP8 GEMM + SwiGLU (quantise, dequantise, fp64 product) on row and column slices of the FFN
+    shape: 512 tokens x K=5120 x 2x1024 output columns per pass."""
+    import torch
+    from oracle.quant import mxfp8_gemm_swiglu
+    g = torch.Generator().manual_seed(5)
+    kdim, rows, cols = CFG_FFN["K"], 512, 1024
+    w = (torch.randn((2 * cols, kdim), generator=g) * 0.02).to(torch.bfloat16)
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        x = torch.randn((rows, kdim), generator=g).to(torch.bfloat16)
+        mxfp8_gemm_swiglu(x, w)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= target_s:
+            break
+    flops = 2.0 * rows * kdim * 2 * cols * passes
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle mxfp8_gemm_swiglu, {passes} passes of {rows} tokens x K={kdim} x 2x{cols} columns "
+                      f"(weights re-quantised every pass, as the oracle does), {dt:.1f} s"}
+
+
 # ---- extras ---------------------------------------------------------------------------------------------
 def extra_dense_1p3b(device, steps, warmup):
     import mindiesd
@@ -356,6 +411,8 @@ def main():
         "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": DENSE_TRAFFIC_BYTES,
+                     "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this launch, scaled by a "
+                                       "1 GiB copy (profiles/fa_fwd_dense_bf16_wan14b_720p.md); not re-measured per run",
                      "kernel": "fa_fwd16_kernel<bf16, 8 waves x 32 rows, 128-key tiles>",
                      "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms},
     }
@@ -376,6 +433,14 @@ def main():
         result["extras"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_dense(cfg)
+        # the same for the other workloads of the path, next to their GPU figures
+        for name, fn in (("sparse_rf_v3", lambda: cpu_baseline_sparse(cfg, device)),
+                         ("mxfp8_gemm_swiglu", cpu_baseline_gemm)):
+            if name in result.get("extras", {}) and "error" not in result["extras"][name]:
+                try:
+                    result["extras"][name]["cpu_baseline"] = fn()
+                except Exception as e:
+                    result["extras"][name]["cpu_baseline"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(result))
 
 

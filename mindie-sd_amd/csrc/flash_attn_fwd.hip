@@ -901,11 +901,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   };
   if constexpr (PAIR) {
     for (int pos = 0; pos < l_n; pos += 2) {
-      const int id_c = pos + 2 < l_n ? __builtin_amdgcn_readfirstlane(l_ptr[pos + 2]) : -1;
-      tile_step(std::integral_constant<int, 0>{}, id_a * BN, id_b >= 0 ? id_b * BN : -1);
-      if (id_b < 0) break;
-      const int id_d = pos + 3 < l_n ? __builtin_amdgcn_readfirstlane(l_ptr[pos + 3]) : -1;
-      tile_step(std::integral_constant<int, 1>{}, id_b * BN, id_c >= 0 ? id_c * BN : -1);
+      const int id_c = __builtin_amdgcn_readfirstlane(l_ptr[pos + 2 < l_n ? pos + 2 : 0]);
+      const int id_d = __builtin_amdgcn_readfirstlane(l_ptr[pos + 3 < l_n ? pos + 3 : 0]);
+      tile_step(std::integral_constant<int, 0>{}, id_a * BN, pos + 1 < l_n ? id_b * BN : -1);
+      if (pos + 1 < l_n) tile_step(std::integral_constant<int, 1>{}, id_b * BN, pos + 2 < l_n ? id_c * BN : -1);
       id_a = id_c;
       id_b = id_d;
     }
