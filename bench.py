@@ -165,6 +165,21 @@ def extra_dense_1p3b(device, steps, warmup):
             "frac_of_bf16_peak": attn_flops(CFG_1P3B) / m / 1e9 / PEAK_BF16_TFLOPS}
 
 
+def extra_head_dims(device, steps, warmup):
+    """Dense attention at head dims other than 128 (the generic kernel): 64 and 256 at a 17776-token sequence."""
+    import torch
+    import mindiesd
+    res = {"workload": "dense bf16 B1 S17776 (13x30x45 latent tokens + 226 text tokens), N48 D64 / N12 D256"}
+    for n, d in ((48, 64), (12, 256)):
+        g = torch.Generator(device=device).manual_seed(7)
+        q, k, v = ((torch.randn((1, n, 17776, d), device=device, generator=g) * 0.5).to(torch.bfloat16) for _ in range(3))
+        ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)
+        m = median(ms)
+        res[f"d{d}_ms"] = m
+        res[f"d{d}_tflops"] = 4.0 * n * 17776 * 17776 * d / m / 1e9
+    return res
+
+
 def extra_causal_varlen(device, steps, warmup):
     """General mode of the dense kernel at the 1.3B shape: bottom-right causal mask (about half of the
     score matrix is skipped) and the same tokens packed as 7 sequences of unequal length."""
@@ -419,6 +434,7 @@ def main():
     if not args.no_extras:
         extras = {}
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
+                         ("head_dims", lambda: extra_head_dims(device, args.steps, args.warmup)),
                          ("causal_varlen", lambda: extra_causal_varlen(device, args.steps, args.warmup)),
                          ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
                          ("ada_bsa", lambda: extra_ada_bsa(device, args.steps, args.warmup, kernel_ms)),

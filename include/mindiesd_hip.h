@@ -9,13 +9,16 @@
  *
  * Return value: 0 on success, otherwise
  *   1  bad argument (null / misaligned pointer, non-positive size, unknown dtype code)
- *   2  unsupported shape or option (head_dim != 128, offsets beyond 32 bits, ...)
+ *   2  unsupported shape or option (head_dim the entry point does not take, offsets beyond 32 bits, ...)
  *   3  workspace too small
  *   4  HIP launch failure
  * (the reference checks the aclnn status the same way: TORCH_CHECK(apiRet == 0, ...),
  * pytorch_npu_helper.h:646-649).
  *
- * dtype codes: 0 = bf16, 1 = fp16.  All tensors have head_dim 128 contiguous in memory; pointers must
+ * dtype codes: 0 = bf16, 1 = fp16.  All tensors have head_dim D contiguous in memory: D = 128 everywhere,
+ * except that the two dense entry points (mindiesd_flash_attention_fwd, mindiesd_flash_attention_general_fwd)
+ * also take every multiple of 8 up to 256 (a generic kernel; the reference's own attention_forward tests run
+ * head_dim 64, tests/layers/flash_attn/test_attn_forward.py:31-169).  Pointers must
  * be 16-byte aligned and every stride a multiple of 8 elements.  "strides" are element strides of the
  * (batch, head, token) dimensions, so BNSD and BSND tensors are both passed without a copy.
  */

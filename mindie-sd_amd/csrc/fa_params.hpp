@@ -1,0 +1,47 @@
+// Argument block shared by the attention kernels of flash_attn_fwd.hip (head_dim 128) and flash_attn_hd.hip
+// (other head dims).
+#pragma once
+#include "common.hpp"
+
+namespace msd {
+
+struct FaParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;  // optional [B, N, Sq] natural-log sum-exp of the scaled scores
+  // element strides of the batch, head and token dimensions (head_dim is contiguous)
+  long long q_sb, q_sn, q_ss;
+  long long k_sb, k_sn, k_ss;
+  long long v_sb, v_sn, v_ss;
+  long long o_sb, o_sn, o_ss;
+  int B, N, Nkv, Sq, Skv;
+  float scale;       // softmax scale
+  float scale_log2;  // scale * log2(e)
+  // block-sparse selection (nullptr => dense): ascending key-block ids per 128-row query block
+  const int* blk_idx;  // [B, N, QB, kb_stride]
+  const int* blk_cnt;  // [B, N, QB]
+  int kb_stride;
+  int QB;
+  const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
+  const int* tok;    // GATHER instantiations: [Sq] row of q/out that holds the token at query position i
+  // two-pass block-sparse attention over paired query blocks (see bsa_pair.hip)
+  const int* pairs;     // PAIR kernel: [B * N][NP][2] query blocks of a pair (second -1: none); lists are per pair
+  int NP;
+  float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)
+  const int* init_cnt;  // second pass: [B * N][QB] key blocks the first pass covered for this query block (0: none)
+  // general mode (MODE = 1 instantiations only)
+  const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
+                              // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count
+  int lse_token_major;        // with seq_meta: lse is [tokens][N] (index (first query token + row) * N + head)
+  int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
+  const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
+  long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
+};
+
+// Dense attention for head dims other than 128 (flash_attn_hd.hip): D a multiple of 8, at most 256; all options of
+// the general mode (packed sequences, causal, boolean mask, lse).
+int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream);
+
+}  // namespace msd

@@ -28,47 +28,13 @@
 #include <utility>
 
 #include "common.hpp"
+#include "fa_params.hpp"
 
 #ifndef FA16_AHEAD
 #define FA16_AHEAD 3  // K operand groups requested ahead of their use in fa_fwd16_kernel
 #endif
 
 namespace msd {
-
-struct FaParams {
-  const void* q;
-  const void* k;
-  const void* v;
-  void* o;
-  float* lse;  // optional [B, N, Sq] natural-log sum-exp of the scaled scores
-  // element strides of the batch, head and token dimensions (head_dim is contiguous)
-  long long q_sb, q_sn, q_ss;
-  long long k_sb, k_sn, k_ss;
-  long long v_sb, v_sn, v_ss;
-  long long o_sb, o_sn, o_ss;
-  int B, N, Nkv, Sq, Skv;
-  float scale;       // softmax scale
-  float scale_log2;  // scale * log2(e)
-  // block-sparse selection (nullptr => dense): ascending key-block ids per 128-row query block
-  const int* blk_idx;  // [B, N, QB, kb_stride]
-  const int* blk_cnt;  // [B, N, QB]
-  int kb_stride;
-  int QB;
-  const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
-  const int* tok;    // GATHER instantiations: [Sq] row of q/out that holds the token at query position i
-  // two-pass block-sparse attention over paired query blocks (see bsa_pair.hip)
-  const int* pairs;     // PAIR kernel: [B * N][NP][2] query blocks of a pair (second -1: none); lists are per pair
-  int NP;
-  float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)
-  const int* init_cnt;  // second pass: [B * N][QB] key blocks the first pass covered for this query block (0: none)
-  // general mode (MODE = 1 instantiations only)
-  const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
-                              // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count
-  int lse_token_major;        // with seq_meta: lse is [tokens][N] (index (first query token + row) * N + head)
-  int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
-  const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
-  long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
-};
 
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
 struct FaCfg {
@@ -987,10 +953,11 @@ using namespace msd;
 extern "C" {
 
 static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
-                        int Nkv, int Sq, int Skv, int D, const long long* st, float scale) {
+                        int Nkv, int Sq, int Skv, int D, const long long* st, float scale, bool any_head_dim = false) {
   if (!q || !k || !v || !out) return MSD_ERR_BAD_ARG;
   if (B <= 0 || N <= 0 || Nkv <= 0 || Sq <= 0 || Skv <= 0 || N % Nkv != 0) return MSD_ERR_BAD_ARG;
-  if (D != 128) return MSD_ERR_UNSUPPORTED;
+  // the dense entry points take head dims 8, 16, ... 256 (flash_attn_hd.hip); everything else is head_dim 128 only
+  if (D != 128 && !(any_head_dim && D > 0 && D <= 256 && (D & 7) == 0)) return MSD_ERR_UNSUPPORTED;
   if (!(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
   // 16-byte vector accesses: every row start must be 16-byte aligned
@@ -999,7 +966,8 @@ static int check_common(const void* q, const void* k, const void* v, const void*
   for (int i = 0; i < 12; ++i) any |= st[i];
   if (any & 7) return MSD_ERR_BAD_ARG;
   // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
-  if ((long long)Skv * st[5] * 2 >= (1ll << 31) || (long long)Skv * st[8] * 2 >= (1ll << 31)) return MSD_ERR_UNSUPPORTED;
+  if (D == 128 && ((long long)Skv * st[5] * 2 >= (1ll << 31) || (long long)Skv * st[8] * 2 >= (1ll << 31)))
+    return MSD_ERR_UNSUPPORTED;
   return MSD_OK;
 }
 
@@ -1115,9 +1083,10 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
                                  long long v_sn, long long v_ss, long long o_sb, long long o_sn, long long o_ss,
                                  float scale, hipStream_t stream) {
   const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
-  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale, true);
   if (rc != MSD_OK) return rc;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16>(p, stream);
   return launch_fa16<MSD_DTYPE_F16>(p, stream);
 }
@@ -1183,7 +1152,7 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
                                          const unsigned char* mask, long long m_sb, long long m_sn, long long m_sq,
                                          hipStream_t stream) {
   const long long st[12] = {q_sb, q_sn, q_ss, k_sb, k_sn, k_ss, v_sb, v_sn, v_ss, o_sb, o_sn, o_ss};
-  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale);
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale, true);
   if (rc != MSD_OK) return rc;
   if (seq_meta && (mask || lse)) return MSD_ERR_UNSUPPORTED;  // packed sequences: neither mask nor lse layout defined
   // m_sq == 0: one mask row shared by all queries (a key-padding mask expanded over the query dimension)
@@ -1191,6 +1160,7 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
+  if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
 }

@@ -12,7 +12,8 @@ from .common import AttentionParam
 from ... import _native
 from ...utils.exception import ParametersInvalid
 
-HEAD_DIM = 128
+HEAD_DIM = 128        # the head_dim of the tuned kernels (sparse, FP8 and the DiT shapes)
+MAX_HEAD_DIM = 256    # dense attention takes every multiple of 8 up to this
 
 
 def _strides_bns(t, layout):
@@ -32,8 +33,9 @@ def _check_qkv(query, key, value):
         raise ParametersInvalid(f"The fused attention kernel supports bf16/fp16 with equal q/k/v dtypes, "
                                 f"but got {query.dtype}, {key.dtype}, {value.dtype}.")
     d = query.shape[-1]
-    if d != HEAD_DIM or key.shape[-1] != d or value.shape[-1] != d:
-        raise ParametersInvalid(f"The fused attention kernel supports head_dim == {HEAD_DIM}, but got {d}.")
+    if d % 8 != 0 or not 0 < d <= MAX_HEAD_DIM or key.shape[-1] != d or value.shape[-1] != d:
+        raise ParametersInvalid(f"The fused attention kernel supports equal q/k/v head_dim, a multiple of 8 up to "
+                                f"{MAX_HEAD_DIM}, but got {d}, {key.shape[-1]}, {value.shape[-1]}.")
 
 
 def _aligned(t):
@@ -165,7 +167,7 @@ class HipFlashAttention(AttentionOperateBase):
 
     @classmethod
     def is_supported_shape(cls, attn_param: AttentionParam) -> bool:
-        return attn_param.head_dim == HEAD_DIM
+        return attn_param.head_dim % 8 == 0 and 0 < attn_param.head_dim <= MAX_HEAD_DIM
 
     @classmethod
     def _run(cls, attn_param, query, key, value, mask, scale):

@@ -123,7 +123,10 @@ def test_dispatch_key_lru_and_registry():
     with pytest.raises(ParametersInvalid):
         get_attention_function(common.AttentionParam(1, 1, 128, 8, 8, torch.float32, True), "hip_flash_attn", "BNSD")
     with pytest.raises(ParametersInvalid):
-        get_attention_function(common.AttentionParam(1, 1, 64, 8, 8, torch.float16, True), "hip_flash_attn", "BNSD")
+        get_attention_function(common.AttentionParam(1, 1, 68, 8, 8, torch.float16, True), "hip_flash_attn", "BNSD")
+    with pytest.raises(ParametersInvalid):
+        get_attention_function(common.AttentionParam(1, 1, 264, 8, 8, torch.float16, True), "hip_flash_attn", "BNSD")
+    get_attention_function(common.AttentionParam(1, 1, 64, 8, 8, torch.float16, True), "hip_flash_attn", "BNSD")
     reg = AttnOpRegistry()
     with pytest.raises(ParametersInvalid):
         reg.register(3, print)
