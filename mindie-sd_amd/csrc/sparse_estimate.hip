@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256) void sbe_select_kernel(const float* scores, si
                                                          int pitch, float threshold, float row_sparse, int keep_sink,
                                                          int keep_recent, int causal) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  extern __shared__ float sh[];  // [NB] row, [NB] sorted
+  extern __shared__ float sh[];  // [NB] row, [NB rounded up to a power of two] sorted
   float* row = sh;
   float* sorted = sh + NB;
   __shared__ float guard_s;
@@ -265,17 +265,26 @@ __global__ __launch_bounds__(256) void sbe_select_kernel(const float* scores, si
   const bool last_out = keep_recent || !causal;
   for (int j = tid; j < L; j += 256) row[j] = ((j == L - 1 && last_out) || (j == 0 && keep_sink)) ? 0.f : src[j];
   __syncthreads();
-  // stable descending rank sort
-  for (int e = tid; e < L; e += 256) {
-    const float x = row[e];
-    int rank = 0;
-    for (int j = 0; j < L; ++j) {
-      const float y = row[j];
-      rank += (y > x || (y == x && j < e)) ? 1 : 0;
-    }
-    sorted[rank] = x;
-  }
+  // descending bitonic sort of the L values, padded with -inf to a power of two (only the sorted values are used,
+  // so the order among equal ones does not matter)
+  int n2 = 1;
+  while (n2 < L) n2 <<= 1;
+  for (int e = tid; e < n2; e += 256) sorted[e] = e < L ? row[e] : -INFINITY;
   __syncthreads();
+  for (int k = 2; k <= n2; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = tid; i < (n2 >> 1); i += 256) {
+        const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1)), hi = lo | j;
+        const float a = sorted[lo], b = sorted[hi];
+        const bool desc = (lo & k) == 0;
+        if (desc ? a < b : a > b) {
+          sorted[lo] = b;
+          sorted[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
   if (tid == 0) {
     float guard = 0.f;
     int cnt = L;
@@ -388,8 +397,11 @@ int mindiesd_sbe_scores(const void* q, const void* k, float* scores, int dtype, 
 int mindiesd_sbe_select(const float* scores, signed char* mask, int* count, int BN, int NB, int pitch, float threshold,
                         float row_sparse, int keep_sink, int keep_recent, int causal, hipStream_t stream) {
   if (!scores || !mask || !count || BN <= 0 || NB <= 0 || pitch < NB) return MSD_ERR_BAD_ARG;
-  if (BN > 65535 || NB * 8 > 60000) return MSD_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(sbe_select_kernel, dim3(NB, BN), dim3(256), NB * 8, stream, scores, mask, count, NB, pitch,
+  int n2 = 1;
+  while (n2 < NB) n2 <<= 1;
+  const int lds = (NB + n2) * 4;
+  if (BN > 65535 || lds > 60000) return MSD_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(sbe_select_kernel, dim3(NB, BN), dim3(256), lds, stream, scores, mask, count, NB, pitch,
                      threshold, row_sparse, keep_sink ? 1 : 0, keep_recent ? 1 : 0, causal ? 1 : 0);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }

@@ -12,7 +12,7 @@ import torch
 from ... import _native
 from ...utils.exception import ParametersInvalid
 from .hip_flash_attn import HEAD_DIM, _strides_bns
-from .rainfusion import BLOCK, _aligned, _check_gpu16, _dims, mask_to_lists
+from .rainfusion import BLOCK, _aligned, _check_gpu16, _dims, block_sparse_attention_mask, mask_to_lists
 
 STRIDE = 8
 # Scratch of the score kernel is allocated up to this size; with more heads than fit, the library goes
@@ -81,6 +81,10 @@ def ada_block_sparse_attention(query, key, value, sparse_mask, sparse_count_tabl
         raise RuntimeError(f"sparse_mask must be [B, N, {nb}, >= {nb}], got {tuple(sparse_mask.shape)}")
     if sparse_count_table is not None and tuple(sparse_count_table.shape) != (b, n, nb):
         raise RuntimeError(f"sparse_count_table must be [B, N, {nb}], got {tuple(sparse_count_table.shape)}")
+    if not causal and q.shape[-1] == HEAD_DIM:
+        # without the in-block causal test this is plain block-sparse attention: the two-pass kernel over paired
+        # query blocks, driven by the mask itself
+        return block_sparse_attention_mask(q, k, v, sparse_mask[..., :nb], scale_value, input_layout)
     idx, cnt = mask_to_lists(sparse_mask)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
