@@ -248,14 +248,22 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
 //   guard -= 1e-5;  column 0 is forced if keep_sink, the last one if keep_recent or not causal;
 //   keep[j] = score[j] > guard;  column 0 is always kept.
 constexpr float kSbeEps = 1e-5f;
+// smallest power of two that is >= n and >= 8
+__host__ __device__ inline int n2_of(int n) {
+  int n2 = 8;
+  while (n2 < n) n2 <<= 1;
+  return n2;
+}
 __global__ __launch_bounds__(256) void sbe_select_kernel(const float* scores, signed char* mask, int* count, int NB,
                                                          int pitch, float threshold, float row_sparse, int keep_sink,
                                                          int keep_recent, int causal) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  extern __shared__ float sh[];  // [NB] row, [NB rounded up to a power of two] sorted
+  extern __shared__ __attribute__((aligned(16))) float sh[];  // [NB] row, [n2] sorted, [n2] running sums (n2: NB rounded up to a power of two, at least 8)
   float* row = sh;
-  float* sorted = sh + NB;
+  float* sorted = sh + ((NB + 3) & ~3);  // 16-byte aligned
+  float* prefix = sorted + n2_of(NB);
   __shared__ float guard_s;
+  __shared__ int first_s;
   __shared__ int cnt_s[4];
   const int tid = threadIdx.x;
   const long long r = (long long)blockIdx.y * NB + blockIdx.x;
@@ -267,8 +275,7 @@ __global__ __launch_bounds__(256) void sbe_select_kernel(const float* scores, si
   __syncthreads();
   // descending bitonic sort of the L values, padded with -inf to a power of two (only the sorted values are used,
   // so the order among equal ones does not matter)
-  int n2 = 1;
-  while (n2 < L) n2 <<= 1;
+  const int n2 = n2_of(L);
   for (int e = tid; e < n2; e += 256) sorted[e] = e < L ? row[e] : -INFINITY;
   __syncthreads();
   for (int k = 2; k <= n2; k <<= 1) {
@@ -285,22 +292,54 @@ __global__ __launch_bounds__(256) void sbe_select_kernel(const float* scores, si
       __syncthreads();
     }
   }
+  // Sequential fp32 running sums of the sorted values (the reference kernel's order of additions), written over
+  // them: one lane, eight values per step from two 16-byte reads that are requested one step ahead (the padding
+  // up to a multiple of 8 holds -inf and only reaches sums past the end, which nobody reads).
+  if (tid == 0 && threshold < 1.0f) {
+    float run = 0.f;
+    f32x4_t a = *(const f32x4_t*)(sorted), b4 = *(const f32x4_t*)(sorted + 4);
+    for (int j = 0; j < L; j += 8) {
+      f32x4_t na = a, nb = b4;
+      if (j + 8 < L) {
+        na = *(const f32x4_t*)(sorted + j + 8);
+        nb = *(const f32x4_t*)(sorted + j + 12);
+      }
+      f32x4_t pa, pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        run += a[i];
+        pa[i] = run;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        run += b4[i];
+        pb[i] = run;
+      }
+      *(f32x4_t*)(prefix + j) = pa;
+      *(f32x4_t*)(prefix + j + 4) = pb;
+      a = na;
+      b4 = nb;
+    }
+  }
+  if (tid == 0) first_s = L - 1;
+  __syncthreads();
+  // first position whose running sum reaches threshold * total (total = the last running sum)
+  if (threshold < 1.0f) {
+    const float lim = threshold * prefix[L - 1];
+    int mine_first = L - 1;
+    for (int j = tid; j < L; j += 256)
+      if (prefix[j] >= lim) {
+        mine_first = j;
+        break;
+      }
+    if (mine_first < L - 1) atomicMin(&first_s, mine_first);
+  }
+  __syncthreads();
   if (tid == 0) {
     float guard = 0.f;
     int cnt = L;
     if (threshold < 1.0f) {
-      float total = 0.f;
-      for (int j = 0; j < L; ++j) total += sorted[j];
-      const float lim = threshold * total;
-      float run = 0.f;
-      cnt = L - 1;
-      for (int j = 0; j < L; ++j) {
-        run += sorted[j];
-        if (run >= lim) {
-          cnt = j;
-          break;
-        }
-      }
+      cnt = first_s;
       guard = sorted[cnt];
     }
     if ((float)cnt > (float)L * row_sparse && L >= 10) {
@@ -397,9 +436,7 @@ int mindiesd_sbe_scores(const void* q, const void* k, float* scores, int dtype, 
 int mindiesd_sbe_select(const float* scores, signed char* mask, int* count, int BN, int NB, int pitch, float threshold,
                         float row_sparse, int keep_sink, int keep_recent, int causal, hipStream_t stream) {
   if (!scores || !mask || !count || BN <= 0 || NB <= 0 || pitch < NB) return MSD_ERR_BAD_ARG;
-  int n2 = 1;
-  while (n2 < NB) n2 <<= 1;
-  const int lds = (NB + n2) * 4;
+  const int lds = (((NB + 3) & ~3) + 2 * n2_of(NB)) * 4;
   if (BN > 65535 || lds > 60000) return MSD_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(sbe_select_kernel, dim3(NB, BN), dim3(256), lds, stream, scores, mask, count, NB, pitch,
                      threshold, row_sparse, keep_sink ? 1 : 0, keep_recent ? 1 : 0, causal ? 1 : 0);
