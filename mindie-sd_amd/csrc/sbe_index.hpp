@@ -14,7 +14,7 @@ namespace msd {
 namespace sbe {
 
 // Geometry.  A strided row / column stands for 8 consecutive tokens; a workgroup owns kTile strided rows and walks
-// the strided columns in tiles of kTile; the head_dim x 8 contraction is walked in 16 chunks of 64 elements
+// a group of strided-column tiles of kTile; the head_dim x 8 contraction is walked in 16 chunks of 64 elements
 // (chunk c: token s = c / 2 of the group of 8, head_dim half dh = c % 2).
 constexpr int kStride = 8;
 constexpr int kTile = 256;                     // strided rows per workgroup = strided columns per tile
@@ -45,11 +45,34 @@ SBE_HD Geom make_geom(int S) {
   return g;
 }
 
-// Workspace per head (floats): partial block sums [Rp][NBp] and the reference maxima they were taken against
-// [Rp][tiles].
+// A row tile's column tiles are split over up to kColGroups workgroups (column groups of nearly equal size), and
+// the workgroups of kRowBlock consecutive row tiles x all column groups are numbered consecutively: the 32
+// workgroups an XCD runs at a time then share 4 query panels (2 MB) and 8 key streams through its L2, where one
+// workgroup per row tile walking all columns had 32 query panels (16 MB) in flight and re-read them from the fabric
+// for every column tile.
+constexpr int kColGroups = 8;
+constexpr int kRowBlock = 4;
+SBE_HD int col_groups(const Geom& g) { return g.tiles < kColGroups ? g.tiles : kColGroups; }
+SBE_HD int group_begin(const Geom& g, int cg) { return (int)((long long)cg * g.tiles / col_groups(g)); }  // cg <= groups
+SBE_HD int work_per_head(const Geom& g) { return g.tiles * col_groups(g); }
+// work item w of a head (0 .. work_per_head - 1) -> row tile and column group
+SBE_HD void decode_work(const Geom& g, int w, int& rt, int& cg) {
+  const int ng = col_groups(g);
+  const int rb = w / (kRowBlock * ng);
+  const int rows_in_block = g.tiles - rb * kRowBlock < kRowBlock ? g.tiles - rb * kRowBlock : kRowBlock;
+  const int within = w - rb * kRowBlock * ng;
+  rt = rb * kRowBlock + within % rows_in_block;
+  cg = within / rows_in_block;
+}
+
+// Workspace per head (floats): partial block sums [Rp][NBp], the reference maxima they were taken against
+// [Rp][tiles], and per row and column group the final maximum and row sum of that group [Rp][kColGroups][2].
 SBE_HD long long part_floats_per_head(const Geom& g) { return (long long)g.Rp * g.NBp; }
 SBE_HD long long mused_floats_per_head(const Geom& g) { return (long long)g.Rp * g.tiles; }
-SBE_HD long long ws_floats_per_head(const Geom& g) { return part_floats_per_head(g) + mused_floats_per_head(g); }
+SBE_HD long long ml_floats_per_head(const Geom& g) { return (long long)g.Rp * kColGroups * 2; }
+SBE_HD long long ws_floats_per_head(const Geom& g) {
+  return part_floats_per_head(g) + mused_floats_per_head(g) + ml_floats_per_head(g);
+}
 
 // Strided columns that the rows of one wave see: all of them, or (causal, the reference's rule
 // tests/plugin/test_sparseblockestimate.py:71-78) those below the end of the wave's step of 1024 query tokens, cut
@@ -94,6 +117,9 @@ SBE_HD long long part_index(const Geom& g, int head_local, int row, int blk) {
 }
 SBE_HD long long mused_index(const Geom& g, int head_local, int row, int tile) {
   return ((long long)head_local * g.Rp + row) * g.tiles + tile;
+}
+SBE_HD long long ml_index(const Geom& g, int head_local, int row, int cg) {
+  return (((long long)head_local * g.Rp + row) * kColGroups + cg) * 2;
 }
 SBE_HD long long score_index(const Geom& g, int head, int brow, int bcol) {
   return ((long long)head * g.NB + brow) * g.NB + bcol;

@@ -10,7 +10,7 @@
 //      query block I puts on 128-token key block J;
 //   3. per query block, sort the key blocks by mass, keep the smallest prefix whose mass reaches `threshold` of
 //      the total (capped at row_sparse * blocks), always keep the first block (attention sink) and the last one.
-// sbe_scores_kernel does 1 and 2 in one pass (P' is never written), sbe_select_kernel does 3.
+// sbe_scores_kernel + sbe_finalize_kernel do 1 and 2 (P' is never written), sbe_select_kernel does 3.
 #include <type_traits>
 
 #include "common.hpp"
@@ -35,22 +35,24 @@ struct SbeParams {
   int causal, col_cap;
   float* part;   // [heads][Rp][NBp]   block sums of exp2(score - reference), per strided row
   float* mused;  // [heads][Rp][tiles] the reference each column tile's sums were taken against
+  float* ml;     // [heads][Rp][kColGroups][2] final maximum and row sum of every column group
   float* scores; // [all heads][NB][NB]
   sbe::Geom g;
 };
 
 // P' as a matrix product: Q' [Sr][8 x 128] (row i = tokens 8i+7, 8i+6, ..., 8i side by side) times K' [Sr][8 x 128]^T
 // (row j = tokens 8j .. 8j+7), i.e. two row-major views of q and k whose 128-wide K chunks are paired in opposite
-// order.  One workgroup (8 waves) owns 256 strided rows (2048 query tokens) of one head and walks the strided
-// columns in tiles of 256; a wave owns 32 rows x 256 columns (8 accumulators of the 32x32x16 instruction, computed
+// order.  One workgroup (8 waves) owns 256 strided rows (2048 query tokens) of one head and walks one group of
+// strided-column tiles of 256 (a row tile's columns are split over up to 8 workgroups, sbe_index.hpp); a wave owns 32 rows x 256 columns (8 accumulators of the 32x32x16 instruction, computed
 // transposed: keys are the rows of the accumulator, so a softmax row lives in one lane pair).  The contraction
 // runs in 16 chunks of 64 elements; a chunk of both operands (2 x 32 KiB) is staged in LDS by LDS-DMA, double
 // buffered, one barrier per chunk.  Tokens past the end of the sequence are outside the buffer descriptors' range
 // and read as zeros, as the reference pads them.
 // After the last chunk of a tile the wave holds the 32 x 256 scores: running row maximum and sum, exp2, sums over
 // the 16 columns of every mask block (8 in-lane additions and one exchange between the wave halves), stored per
-// strided row together with the maximum they refer to.  When all tiles are done the wave reads its rows back,
-// rescales them to the final maximum, divides by the row sum and adds up the 16 rows of each mask block.
+// strided row together with the maximum they refer to.  When its tiles are done the workgroup stores the maximum and
+// row sum its column group ended with; sbe_finalize_kernel combines the groups, rescales the stored sums to the final
+// maximum, divides by the row sum and adds up the 16 rows of each mask block.
 template <int DT>
 __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -65,13 +67,15 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
   const int l32 = lane & 31, h = lane >> 5;
   const Geom g = p.g;
 
-  // consecutive row tiles of one head stay on one XCD (they stream the same keys through its L2)
-  const int total = p.heads * g.tiles;
+  // consecutive work items stay on one XCD: 4 row tiles x 8 column groups of one head at a time (decode_work)
+  const int wph = work_per_head(g);
+  const int total = p.heads * wph;
   const int per_xcd = (total + 7) / 8;
   const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if ((int)(blockIdx.x >> 3) >= per_xcd || work >= total) return;
-  const int hl = work / g.tiles;                       // head inside this launch
-  int rt = work - hl * g.tiles;
+  const int hl = work / wph;                           // head inside this launch
+  int rt, cg;
+  decode_work(g, work - hl * wph, rt, cg);
   if (p.causal) rt = g.tiles - 1 - rt;                 // the row tiles with the most columns start first
   const int head = p.head0 + hl;
   const int b = head / p.N, n = head - b * p.N;
@@ -87,7 +91,10 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
   const int q_voff = dma_voffset(wave, lane, p.q_ss), k_voff = dma_voffset(wave, lane, p.k_ss);
 
   const int my_cols = wave_cols(g, p.causal, p.col_cap, i0 + 32 * wave);  // strided columns this wave's rows see
-  const int n_tiles = wg_col_tiles(g, p.causal, p.col_cap, i0);
+  // this workgroup's column tiles: its group, cut at the last tile any of its rows sees
+  const int t_begin = group_begin(g, cg);
+  const int t_end = min(group_begin(g, cg + 1), wg_col_tiles(g, p.causal, p.col_cap, i0));
+  if (t_begin >= t_end) return;
 
   // chunk c of column tile t into LDS stage `stage`: query rows i0.., token 7 - s; key columns 256 t.., token s
   auto load_chunk = [&](int t, int s, int dh, int stage) {
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
   float* part_row = p.part + part_index(g, hl, my_row, 0);
   float* mused_row = p.mused + mused_index(g, hl, my_row, 0);
 
-  load_chunk(0, 0, 0, 0);
+  load_chunk(t_begin, 0, 0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
@@ -144,14 +151,14 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
     __syncthreads();
   };
 
-  for (int t = 0; t < n_tiles; ++t) {
+  for (int t = t_begin; t < t_end; ++t) {
 #pragma unroll
     for (int kb = 0; kb < 8; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[kb][r] = 0.f;
     for (int s = 0; s < kStride; ++s) {
       chunk_step(std::integral_constant<int, 0>{}, t, s, true, t, s);
-      const bool more = s + 1 < kStride || t + 1 < n_tiles;
+      const bool more = s + 1 < kStride || t + 1 < t_end;
       chunk_step(std::integral_constant<int, 1>{}, t, s, more, s + 1 < kStride ? t : t + 1, s + 1 < kStride ? s + 1 : 0);
     }
 
@@ -178,7 +185,7 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[kb][r]);
       mx = half_max(mx) * p.scale_log2;  // at least one column of the tile is visible, so this is finite
       const float m_new = fmaxf(m_run, mx);
-      l_run *= fast_exp2(m_run - m_new);  // first tile: exp2(-inf) = 0
+      l_run *= fast_exp2(m_run - m_new);  // first visible tile: exp2(-inf) = 0
       m_run = m_new;
 #pragma unroll
       for (int kb = 0; kb < 8; ++kb) {
@@ -205,32 +212,52 @@ __global__ __launch_bounds__(512, 1) void sbe_scores_kernel(const SbeParams p) {
     if (h == 0) mused_row[t] = m_run;
   }
 
-  // ---- block scores of this wave's two block rows ------------------------------------------------------------
+  // ---- the group's final maximum and row sum (-inf and 0 for rows that saw none of its columns) ---------------------
   const float l_tot = half_sum(l_run);
-  const float inv_l = 1.0f / l_tot;
-  __threadfence_block();
-  __syncthreads();  // the rows written above are read back by other lanes of the same wave
+  if (h == 0) *(f32x2_t*)(p.ml + ml_index(g, hl, my_row, cg)) = f32x2_t{m_run, l_tot};
+#endif
+}
+
+// Second step of the block scores: one workgroup of 64 lanes per (head, mask block row).  For each of its (up to)
+// 16 strided rows the final maximum and row sum are put together from the column groups, then lane J adds up the
+// rows' sums of block J, each brought from the reference it was taken against to the final one and divided by the
+// row sum.  Columns past the last tile the row tile walked (causal) are zero.
+__global__ __launch_bounds__(64) void sbe_finalize_kernel(const SbeParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  using namespace sbe;
+  const Geom g = p.g;
+  const int lane = threadIdx.x;
+  const int brow = blockIdx.x, hl = blockIdx.y;
+  const int head = p.head0 + hl;
+  const int row0 = 16 * brow;
+  const int rows = min(16, g.Sr - row0);  // > 0 because brow < NB
+  const int i0 = row0 / kTile * kTile;
+  const int n_tiles = wg_col_tiles(g, p.causal, p.col_cap, i0);
+  const int ng = col_groups(g);
+  // lane i < rows: final maximum and reciprocal row sum of row row0 + i
+  float m_fin = -INFINITY, inv_l = 0.f;
+  if (lane < rows) {
+    const float* ml = p.ml + ml_index(g, hl, row0 + lane, 0);
+    for (int c = 0; c < ng && group_begin(g, c) < n_tiles; ++c) m_fin = fmaxf(m_fin, ml[2 * c]);
+    float l = 0.f;
+    for (int c = 0; c < ng && group_begin(g, c) < n_tiles; ++c) l += ml[2 * c + 1] * fast_exp2(ml[2 * c] - m_fin);
+    inv_l = 1.0f / l;
+  }
   const int blocks_done = n_tiles * kBlocksPerTile;
-  for (int br = 0; br < 2; ++br) {
-    const int brow = (i0 + 32 * wave) / 16 + br;
-    if (brow >= g.NB) break;
-    const int row0 = i0 + 32 * wave + 16 * br;
-    const int rows = min(16, g.Sr - row0);  // > 0 because brow < NB
-    float* out = p.scores + score_index(g, head, brow, 0);
-    for (int J0 = 0; J0 < g.NB; J0 += 64) {
-      const int J = J0 + lane;
-      const bool live = J < g.NB && J < blocks_done;
-      const float* pr = p.part + part_index(g, hl, row0, live ? J : 0);
-      const float* mr = p.mused + mused_index(g, hl, row0, live ? J >> 4 : 0);
-      float v = 0.f;
+  float* out = p.scores + score_index(g, head, brow, 0);
+  for (int J0 = 0; J0 < g.NB; J0 += 64) {
+    const int J = J0 + lane;
+    const bool live = J < g.NB && J < blocks_done;
+    const float* pr = p.part + part_index(g, hl, row0, live ? J : 0);
+    const float* mr = p.mused + mused_index(g, hl, row0, live ? J >> 4 : 0);
+    float v = 0.f;
 #pragma unroll 1
-      for (int i = 0; i < rows; ++i) {  // wave-uniform trip count and lane index
-        const float m_fin = lane_value(m_run, 16 * br + i);
-        const float w = lane_value(inv_l, 16 * br + i);
-        v += pr[(long long)i * g.NBp] * fast_exp2(mr[i * g.tiles] - m_fin) * w;
-      }
-      if (J < g.NB) out[J] = live ? v : 0.f;
+    for (int i = 0; i < rows; ++i) {  // wave-uniform trip count and lane index
+      const float mf = lane_value(m_fin, i);
+      const float w = lane_value(inv_l, i);
+      v += pr[(long long)i * g.NBp] * fast_exp2(mr[i * g.tiles] - mf) * w;
     }
+    if (J < g.NB) out[J] = live ? v : 0.f;
   }
 #endif
 }
@@ -420,12 +447,14 @@ int mindiesd_sbe_scores(const void* q, const void* k, float* scores, int dtype, 
     p.col_cap = S / sbe::kStride > 0 ? S / sbe::kStride : 1;
     p.part = (float*)workspace;
     p.mused = p.part + (long long)p.heads * sbe::part_floats_per_head(g);
+    p.ml = p.mused + (long long)p.heads * sbe::mused_floats_per_head(g);
     p.scores = scores;
     p.g = g;
-    const long long total = (long long)p.heads * g.tiles;
-    if (total > (1ll << 30)) return MSD_ERR_UNSUPPORTED;
+    const long long total = (long long)p.heads * sbe::work_per_head(g);
+    if (total > (1ll << 30) || p.heads > 65535) return MSD_ERR_UNSUPPORTED;
     const unsigned grid = (unsigned)((total + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), sbe::kLdsBytes, stream, p);
+    hipLaunchKernelGGL(sbe_finalize_kernel, dim3(g.NB, p.heads), dim3(64), 0, stream, p);
     if (hipGetLastError() != hipSuccess) return MSD_ERR_LAUNCH;
   }
   return MSD_OK;
