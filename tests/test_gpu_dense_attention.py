@@ -135,7 +135,7 @@ def test_errors(cuda):
     with pytest.raises(ParametersInvalid):
         mindiesd.attention_forward(q.float(), q.float(), q.float())
     with pytest.raises(ParametersInvalid):
-        mindiesd.attention_forward(q[..., :64], q[..., :64], q[..., :64])
+        mindiesd.attention_forward(q[..., :68], q[..., :68], q[..., :68])   # head_dim must be a multiple of 8
     with pytest.raises(ParametersInvalid):
         mindiesd.attention_forward(q, q, q, opt_mode="manual", op_type="nope")
 
