@@ -442,7 +442,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         // first tile: move to the exact row maximum (delta may be negative); later: only upwards
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
-        const float alpha = fast_exp2(-delta);
+        // (first tile: sums and outputs are still zero; 2^-delta would overflow for rows far below zero and 0 * inf is NaN)
+        const float alpha = first ? 1.f : fast_exp2(-delta);
         m_run[qb] += delta;
         l_run[qb] *= alpha;
 #pragma unroll
@@ -805,7 +806,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
         mx = quarter_max(mx);
         delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
-        alpha = fast_exp2(-delta);
+        // (first tile: sums and outputs are still zero; 2^-delta would overflow for rows far below zero and 0 * inf is NaN)
+        alpha = first ? 1.f : fast_exp2(-delta);
         moved = 1;
       }
       // the rescale itself: in place, skipped when the reference did not move (see cond_rescale_fa16)

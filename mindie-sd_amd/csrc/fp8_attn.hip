@@ -525,7 +525,8 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
         mx = half_max(mx);
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
-        const float alpha = fast_exp2(-delta);
+        // (first tile: sums and outputs are still zero; 2^-delta would overflow for rows far below zero and 0 * inf is NaN)
+        const float alpha = first ? 1.f : fast_exp2(-delta);
         m_run += delta;
 #pragma unroll
         for (int r = 0; r < 16; ++r) negm[r] = kPShift - m_run;

@@ -176,7 +176,8 @@ def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2):
                         mx = s.max(axis=1) - m_run
                         if first or (mx > P_TAU).any():
                             delta = mx if first else np.maximum(mx, np.float32(0))
-                            alpha = np.exp2(-delta).astype(np.float32)
+                            # (first tile: sums and outputs are still zero, the factor is 1; 2^-delta may overflow)
+                            alpha = np.ones_like(delta) if first else np.exp2(-delta).astype(np.float32)
                             m_run = m_run + delta
                             l_run *= alpha
                             o_run *= alpha[:, None]

@@ -53,6 +53,28 @@ def test_paired_vs_oracle_and_lists(cuda, s, n, nkv, dtype):
     assert (lse[rows] - lse1[rows]).abs().max().item() < 5e-3
 
 
+def test_paired_scores_far_below_zero(cuda):
+    """Every score hundreds of units below zero (q = +8, k near -8): the first key block of a row moves the running
+    maximum far down in both passes.  (Constant queries: the kernel's rounding of q * scale * log2(e) to bf16 is then a
+    common factor of all scores, which at |s| ~ 700 would otherwise exceed the tolerance.)"""
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    s, n = 1100, 2
+    g = torch.Generator().manual_seed(11)
+    q = torch.full((1, n, s, 128), 8.0, dtype=torch.bfloat16)
+    k = (-8.0 + 0.5 * torch.randn((1, n, s, 128), generator=g)).to(torch.bfloat16)
+    v = torch.randn((1, n, s, 128), generator=g).to(torch.bfloat16)
+    nb = (s + 127) // 128
+    m = _banded_mask(1, n, nb, nb, seed=12)
+    want = oa.block_sparse_attention(q, k, v, m.numpy())
+    out = rf.block_sparse_attention_mask(q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda), 128 ** -0.5, "BNSD")
+    assert not torch.isnan(out.float()).any()
+    eb, ok, mx = oa.ref_compare(want, out.cpu(), 2.0 ** -6)
+    assert ok, (eb, mx)
+    idx, cnt = rf.mask_to_lists(m.to(torch.int8).to(cuda))
+    out1 = rf.block_sparse_attention_lists(q.to(cuda), k.to(cuda), v.to(cuda), idx, cnt, 128 ** -0.5, "BNSD")
+    assert oa.ref_compare(want, out1.cpu(), 2.0 ** -6)[1]
+
+
 def test_paired_bsnd_cross_lengths_and_full_mask(cuda):
     """BSND tensors in place, more keys than queries, and the all-ones mask (= dense attention)."""
     from mindiesd.layers.flash_attn import rainfusion as rf

@@ -100,6 +100,33 @@ def test_rising_row_maxima_vs_fp64(cuda):
         _check(out[0, n], ref, max_abs=1e-1)
 
 
+def _far_below_zero(shape, seed, dtype=torch.bfloat16):
+    """q near +8, k near -8 in every component: every score of a row lies hundreds of units below zero, so the first
+    key tile already moves the running maximum far down (2^-delta overflows there); v is N(0, 1)."""
+    g = torch.Generator().manual_seed(seed)
+    q = (8.0 + 0.5 * torch.randn(shape, generator=g)).to(dtype)
+    k = (-8.0 + 0.5 * torch.randn(shape, generator=g)).to(dtype)
+    v = torch.randn(shape, generator=g).to(dtype)
+    return q, k, v
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("s", [300, 1153])
+def test_scores_far_below_zero(cuda, s, d):
+    """Checked against an fp64 evaluation on the queries as the kernel uses them (scaled by scale * log2(e) and
+    rounded to bf16, the reference rounds q * scale as well, attention_func.py:40): at |s| ~ 700 the bf16-rounded
+    scores of the reference's unfused path are too coarse to serve as the yardstick."""
+    import math
+    import mindiesd
+    from oracle.attention import attention_fp64
+    q, k, v = _far_below_zero((1, 2, s, d), seed=s + d)
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
+    assert not torch.isnan(out.float()).any()
+    qs = (q.float() * (d ** -0.5 * math.log2(math.e))).to(torch.bfloat16)
+    for n in range(2):
+        _check(out[0, n], attention_fp64(qs[0, n], k[0, n], v[0, n], math.log(2.0)))
+
+
 def test_config2_head_subset(cuda):
     """Wan2.1-1.3B shape (S=32760): full GPU run, oracle on a row sample of two heads."""
     import mindiesd

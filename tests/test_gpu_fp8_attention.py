@@ -121,6 +121,22 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
     assert err_m.max() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("recipe", ["pow2", "amax"])
+def test_fp8_attention_scores_far_below_zero(cuda, recipe):
+    """q near +8, k near -8: every score lies hundreds of units below zero, the first key tile moves the running
+    maximum far down."""
+    from mindiesd.layers.quant import fp8_attention_forward
+    g = torch.Generator().manual_seed(21)
+    shape = (1, 2, 1100, 128)
+    q = (8.0 + 0.5 * torch.randn(shape, generator=g)).to(torch.bfloat16)
+    k = (-8.0 + 0.5 * torch.randn(shape, generator=g)).to(torch.bfloat16)
+    v = torch.randn(shape, generator=g).to(torch.bfloat16)
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True)
+    out = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), layout="BNSD", recipe=recipe).cpu()
+    assert not torch.isnan(out.float()).any()
+    assert cosine(out, want) >= 0.999
+
+
 @pytest.mark.parametrize("layout,dtype", [("BNSD", torch.bfloat16), ("BSND", torch.bfloat16), ("BNSD", torch.float16)])
 def test_rotation_fused_into_block_quant(cuda, layout, dtype):
     """x @ rot -> 16-bit -> block quantisation in one kernel vs matmul + quantisation on the CPU.  The two
