@@ -334,6 +334,9 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
   bool first = !resumed;  // no tile has been folded into this wave's running softmax yet
+  bool unseen[C::kNQB];   // general mode: this lane's row has not met a visible key yet
+#pragma unroll
+  for (int qb = 0; qb < C::kNQB; ++qb) unseen[qb] = true;
 
   // One tile step: fetch the tile at next_key0 (< 0: none) into the other stage, compute on the tile
   // at key0 if this wave takes part in it.  The LDS stage is a compile-time constant (the loops
@@ -437,13 +440,18 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][qb][r]);
       // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
-      if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+      // General mode: a mask can hide a whole tile from a row, so "nothing folded in yet" is kept per row - a row
+      // takes its exact maximum as reference with the first tile that shows it a key, whichever tile that is.
+      const bool lane_wants = MODE ? (mx > kTau || (unseen[qb] && mx > -INFINITY)) : mx > kTau;
+      if ((!MODE && first) || __builtin_amdgcn_ballot_w64(lane_wants) != 0) {
         mx = half_max(mx);
-        // first tile: move to the exact row maximum (delta may be negative); later: only upwards
-        float delta = first ? mx : fmaxf(mx, 0.f);
+        const bool fresh = MODE ? unseen[qb] : first;
+        // first visible tile: move to the exact row maximum (delta may be negative); later: only upwards
+        float delta = fresh ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
         // (first tile: sums and outputs are still zero; 2^-delta would overflow for rows far below zero and 0 * inf is NaN)
-        const float alpha = first ? 1.f : fast_exp2(-delta);
+        const float alpha = fresh ? 1.f : fast_exp2(-delta);
+        if (MODE) unseen[qb] = unseen[qb] && mx == -INFINITY;
         m_run[qb] += delta;
         l_run[qb] *= alpha;
 #pragma unroll

@@ -53,6 +53,25 @@ def test_sparse_block_estimate_vs_oracle(cuda, s, threshold, row_sparse, dtype):
         _mask_close(got[0, h], want[0, h])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("sign", [-1.0, 1.0, 0.0])
+def test_estimate_on_scores_far_from_zero(cuda, sign, dtype):
+    """q near +8 and k near -8 / +8 (every strided score hundreds of units below / above zero), and all-zero inputs
+    (uniform rows): the running maxima of the score kernel start from nothing in every case."""
+    import mindiesd  # noqa: F401
+    g = torch.Generator().manual_seed(5)
+    q = ((8.0 + 0.5 * torch.randn((1, 2, 2048, 128), generator=g)) * abs(sign)).to(dtype)
+    k = ((8.0 * sign + 0.5 * torch.randn((1, 2, 2048, 128), generator=g)) * abs(sign)).to(dtype)
+    smask, sct = torch.ops.mindiesd.sparse_block_estimate(
+        q.to(cuda), k.to(cuda), input_layout="BNSD", stride=8, sparse_size=128, num_heads=2, num_key_value_heads=2,
+        scale_value=128 ** -0.5 / 8, threshold=0.85, causal=False, keep_sink=True, keep_recent=True, row_sparse=1.0)
+    got = smask.cpu().numpy().astype(bool)
+    assert np.array_equal(sct.cpu().numpy(), got.sum(-1))
+    want = oab.sparse_estimate(q, k, threshold=0.85, force_sparse=1.0, rules="kernel")
+    for h in range(2):
+        _mask_close(got[0, h, :, :16], want[0, h])
+
+
 def test_estimate_against_the_numpy_statement_on_the_reference_test_case(cuda):
     """The reference's own test (tests/plugin/test_sparseblockestimate.py:150-241): B1 N1 S8192 D128, N(0,1) inputs
     cast to fp16, threshold 0.85, no cap, default switches, kernel against the numpy statement within 2 % / 1 %."""

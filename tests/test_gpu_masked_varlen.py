@@ -40,6 +40,27 @@ def test_fused_attention_with_boolean_mask(cuda, mask_shape, head_first):
     _check(out if head_first else out.transpose(1, 2), ref)
 
 
+def test_mask_hides_the_first_tiles_and_scores_lie_far_below_zero(cuda):
+    """Block-diagonal mask (rows of the second half see keys of the second half only, so their first two key tiles are
+    hidden) on scores hundreds of units below zero: a row must take its reference maximum from the first tile that
+    shows it a key.  fp64 yardstick on the queries as the kernel rounds them (q * scale * log2(e) in bf16)."""
+    import math
+    import mindiesd
+    from oracle.attention import attention_fp64
+    s = 600
+    g = torch.Generator().manual_seed(9)
+    q = (8.0 + 0.5 * torch.randn((1, 2, s, 128), generator=g)).to(torch.bfloat16)
+    k = (-8.0 + 0.5 * torch.randn((1, 2, s, 128), generator=g)).to(torch.bfloat16)
+    v = torch.randn((1, 2, s, 128), generator=g).to(torch.bfloat16)
+    mask = torch.zeros(s, s, dtype=torch.bool)
+    mask[:300, :300] = True
+    mask[300:, 300:] = True
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=mask.to(cuda), head_first=True).cpu()
+    qs = (q.float() * (128 ** -0.5 * math.log2(math.e))).to(torch.bfloat16)
+    for n in range(2):
+        _check(out[0, n], attention_fp64(qs[0, n], k[0, n], v[0, n], math.log(2.0), keep=mask.numpy()))
+
+
 def test_mask_dtypes_and_fully_masked_rows(cuda):
     from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
     q, k, v = _rand((1, 2, 130, 128), 5), _rand((1, 2, 200, 128), 6), _rand((1, 2, 200, 128), 7)
