@@ -39,6 +39,8 @@ def window_order(t, h, w):
         return ids.reshape(t, h // 8, 8, w // 8, 8).transpose(0, 1, 3, 2, 4).reshape(-1)
     h8, w8 = h - h % 8, w - w % 8
     first = ids[: h * w]
+    if t == 1:  # a single frame: nothing follows the frame that stays in place
+        return first
     grid = ids[h * w:].reshape(t - 1, h, w)
     parts = [grid[:, :h8, :w8].reshape(t - 1, h8 // 8, 8, w8 // 8, 8).transpose(0, 1, 3, 2, 4).reshape(t - 1, -1)]
     if h % 8:

@@ -1,0 +1,91 @@
+"""GPU parity on shapes drawn at random (fixed seeds): sequence lengths around every tile and block boundary, unequal
+query / key lengths, grouped-query heads, both layouts and dtypes, head dims of every kernel, random boolean masks,
+causal masks and random block masks, each against the CPU oracle with the tolerance of the path's own test file."""
+import random
+
+import pytest
+import torch
+
+from oracle import attention as oa
+from oracle.attention import attention_math, causal_keep_mask
+
+pytestmark = pytest.mark.gpu
+
+SQ = [1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 127, 129, 255, 256, 257, 383, 385, 511, 513, 640, 777, 1000]
+SKV = [1, 3, 32, 63, 64, 65, 96, 127, 128, 129, 191, 193, 255, 257, 300, 449, 512, 515, 901]
+
+
+def _rnd(shape, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g).to(dtype)
+
+
+def _heads(r):
+    n = r.choice([1, 2, 3, 4])
+    return n, r.choice([x for x in (1, 2, 3, 4) if n % x == 0])
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_dense_random_shape(cuda, seed):
+    import mindiesd
+    r = random.Random(seed)
+    d = r.choice([128, 128, 64, 32, 96, 256])
+    sq = r.choice(SQ)
+    skv = sq if r.random() < 0.5 else r.choice(SKV)
+    (n, nkv), b = _heads(r), r.choice([1, 2])
+    dtype, hf = r.choice([torch.bfloat16, torch.float16]), r.random() < 0.5
+    q, k, v = _rnd((b, n, sq, d), seed, dtype), _rnd((b, nkv, skv, d), seed + 1000, dtype), _rnd((b, nkv, skv, d), seed + 2000, dtype)
+    ref = attention_math(q, k.repeat_interleave(n // nkv, 1), v.repeat_interleave(n // nkv, 1), None, d ** -0.5, head_first=True)
+    args = (q, k, v) if hf else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = mindiesd.attention_forward(*(t.to(cuda) for t in args), head_first=hf).cpu()
+    out = out if hf else out.transpose(1, 2)
+    assert not torch.isnan(out.float()).any()
+    assert (out.float() - ref.float()).abs().max().item() <= 2e-2, (b, n, nkv, sq, skv, d, dtype, hf)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_masked_or_causal_random_shape(cuda, seed):
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    r = random.Random(100 + seed)
+    d = r.choice([128, 128, 64])
+    sq, skv = r.choice([1, 17, 64, 100, 129, 256, 300, 513]), r.choice([1, 5, 64, 65, 128, 200, 257, 400, 640])
+    (n, nkv), b = _heads(r), r.choice([1, 2])
+    causal = r.random() < 0.4
+    q, k, v = _rnd((b, n, sq, d), seed, torch.bfloat16), _rnd((b, nkv, skv, d), seed + 1, torch.bfloat16), _rnd((b, nkv, skv, d), seed + 2, torch.bfloat16)
+    if causal:
+        mask, keep = None, causal_keep_mask(sq, skv)[None, None].expand(b, n, sq, skv)
+    else:
+        g = torch.Generator().manual_seed(seed)
+        mask = torch.rand((b, r.choice([1, n]), sq, skv), generator=g) > r.choice([0.2, 0.5, 0.9])
+        keep = mask.expand(b, n, sq, skv)
+    ref = attention_math(q, k.repeat_interleave(n // nkv, 1), v.repeat_interleave(n // nkv, 1), keep, d ** -0.5, head_first=True)
+    ref = torch.where(keep.any(-1)[..., None], ref, torch.zeros((), dtype=ref.dtype))  # rows without a visible key: zeros
+    out = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BNSD",
+                          attn_mask=None if mask is None else mask.to(cuda), causal=causal).cpu()
+    assert not torch.isnan(out.float()).any()
+    # A row that sees only a handful of keys is a weighted mean of a few v rows: the rounding of the scores (the
+    # reference keeps q * scale and q k^T in bf16, attention_func.py:40-41, the kernel q * scale * log2(e)) moves
+    # single weights by a few per cent and nothing averages that out, hence 5e-2 where the dense bound is 2e-2.
+    err = (out.float() - ref.float()).abs()
+    assert bool((err <= 5e-2 * ref.float().abs().clamp(min=1.0)).all()), (err.max().item(), b, n, nkv, sq, skv, d, causal)
+    dense_rows = keep.sum(-1) >= 32
+    assert err[dense_rows].max().item() <= 2e-2 if dense_rows.any() else True
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_block_sparse_random_mask(cuda, seed):
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    r = random.Random(200 + seed)
+    s = r.choice([130, 255, 256, 257, 500, 640, 769, 1024, 1100, 1537])
+    n = r.choice([1, 2, 4])
+    nkv, b = r.choice([x for x in (1, 2, 4) if n % x == 0]), r.choice([1, 2])
+    dtype = r.choice([torch.bfloat16, torch.float16])
+    q, k, v = _rnd((b, n, s, 128), seed, dtype), _rnd((b, nkv, s, 128), seed + 1, dtype), _rnd((b, nkv, s, 128), seed + 2, dtype)
+    nb = (s + 127) // 128
+    g = torch.Generator().manual_seed(seed)
+    m = torch.rand(b, n, nb, nb, generator=g) < r.choice([0.1, 0.3, 0.6, 0.9])
+    want = oa.block_sparse_attention(q, k, v, m.numpy())
+    out = rf.block_sparse_attention_mask(q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda), 128 ** -0.5, "BNSD").cpu()
+    assert not torch.isnan(out.float()).any()
+    eb, ok, mx = oa.ref_compare(want, out, 2.0 ** -6)
+    assert ok, (eb, mx, b, n, nkv, s, dtype)
