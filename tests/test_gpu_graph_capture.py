@@ -1,0 +1,65 @@
+"""The entry points enqueue on the current stream and never synchronise, so a caller can capture them in a HIP graph
+(torch.cuda.CUDAGraph).  Every replay is checked against the eager result, with eager work and synchronisations of
+the program between the replays."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _rnd(shape, seed, dtype=torch.bfloat16, mul=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * mul).to(dtype)
+
+
+def _capture_and_replay(cuda, fn, inputs, fresh_inputs):
+    """fn(*inputs) -> tensor.  Captures fn on static input buffers, then replays it three times on new input values."""
+    static = [t.clone() for t in inputs]
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(side):
+        for _ in range(2):  # warm-up outside the capture (library loading, kernel attributes)
+            fn(*static)
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    torch.cuda.synchronize(cuda)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn(*static)
+    for step, new in enumerate(fresh_inputs):
+        for dst, src in zip(static, new):
+            dst.copy_(src)
+        graph.replay()
+        got = out.clone()
+        want = fn(*[t.clone() for t in new])          # eager work between the replays
+        torch.cuda.synchronize(cuda)
+        assert torch.equal(got, want), f"replay {step} differs from the eager call"
+
+
+def test_dense_attention_in_a_graph(cuda):
+    import mindiesd
+    mk = lambda s: tuple(_rnd((1, 4, 700, 128), s + i).to(cuda) for i in range(3))
+    _capture_and_replay(cuda, lambda q, k, v: mindiesd.attention_forward(q, k, v, head_first=True), mk(0), [mk(10), mk(20), mk(30)])
+
+
+def test_fp8_attention_in_a_graph(cuda):
+    from mindiesd.layers.quant import fp8_attention_forward
+    mk = lambda s: tuple(_rnd((1, 2, 900, 128), s + i).to(cuda) for i in range(3))
+    _capture_and_replay(cuda, lambda q, k, v: fp8_attention_forward(q, k, v, layout="BNSD", recipe="amax"), mk(0), [mk(10), mk(20), mk(30)])
+
+
+def test_mxfp8_gemm_swiglu_in_a_graph(cuda):
+    from mindiesd.layers.quant import mx_quantize, mxfp8_gemm_swiglu
+    wq, ws = mx_quantize(_rnd((2 * 264, 512), 5, mul=0.05).to(cuda))
+    mk = lambda s: (_rnd((300, 512), s).to(cuda),)
+    _capture_and_replay(cuda, lambda x: mxfp8_gemm_swiglu(x, wq, ws), mk(0), [mk(10), mk(20), mk(30)])
+
+
+def test_block_sparse_attention_in_a_graph(cuda):
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    s, n = 1100, 2
+    nb = (s + 127) // 128
+    g = torch.Generator().manual_seed(3)
+    mask = (torch.rand(1, n, nb, nb, generator=g) < 0.4).to(torch.int8).to(cuda)
+    mk = lambda sd: tuple(_rnd((1, n, s, 128), sd + i).to(cuda) for i in range(3))
+    _capture_and_replay(cuda, lambda q, k, v: rf.block_sparse_attention_mask(q, k, v, mask, 128 ** -0.5, "BNSD"),
+                        mk(0), [mk(10), mk(20), mk(30)])
