@@ -63,3 +63,42 @@ def test_block_sparse_attention_in_a_graph(cuda):
     mk = lambda sd: tuple(_rnd((1, n, s, 128), sd + i).to(cuda) for i in range(3))
     _capture_and_replay(cuda, lambda q, k, v: rf.block_sparse_attention_mask(q, k, v, mask, 128 ** -0.5, "BNSD"),
                         mk(0), [mk(10), mk(20), mk(30)])
+
+
+def test_two_streams_and_two_threads(cuda):
+    """Launches from two host threads on two streams at once (no shared state in the library): each result equals the
+    one computed alone."""
+    import threading
+    import mindiesd
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    s, n = 900, 2
+    nb = (s + 127) // 128
+    g = torch.Generator().manual_seed(4)
+    mask = (torch.rand(1, n, nb, nb, generator=g) < 0.5).to(torch.int8).to(cuda)
+    inputs = [tuple(_rnd((1, n, s, 128), 40 * t + i).to(cuda) for i in range(3)) for t in range(2)]
+    alone = [(mindiesd.attention_forward(*x, head_first=True), rf.block_sparse_attention_mask(*x, mask, 128 ** -0.5, "BNSD"))
+             for x in inputs]
+    torch.cuda.synchronize(cuda)
+    results, errors = [None, None], []
+
+    def work(t):
+        try:
+            st = torch.cuda.Stream(device=cuda)
+            with torch.cuda.stream(st):
+                outs = []
+                for _ in range(8):
+                    outs = (mindiesd.attention_forward(*inputs[t], head_first=True),
+                            rf.block_sparse_attention_mask(*inputs[t], mask, 128 ** -0.5, "BNSD"))
+                st.synchronize()
+            results[t] = outs
+        except Exception as e:  # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for t in range(2):
+        assert torch.equal(results[t][0], alone[t][0]) and torch.equal(results[t][1], alone[t][1])
