@@ -1,6 +1,8 @@
 """GPU parity on shapes drawn at random (fixed seeds): sequence lengths around every tile and block boundary, unequal
 query / key lengths, grouped-query heads, both layouts and dtypes, head dims of every kernel, random boolean masks,
-causal masks and random block masks, each against the CPU oracle with the tolerance of the path's own test file."""
+causal masks and random block masks, each against the CPU oracle with the tolerance of the path's own test file;
+the two quantisers bit for bit on values spread over many octaves, tiny values, values on a coarse grid (rounding
+ties) and outliers."""
 import random
 
 import pytest
@@ -89,3 +91,55 @@ def test_block_sparse_random_mask(cuda, seed):
     assert not torch.isnan(out.float()).any()
     eb, ok, mx = oa.ref_compare(want, out, 2.0 ** -6)
     assert ok, (eb, mx, b, n, nkv, s, dtype)
+
+
+def _values(shape, seed, dtype, kind):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g)
+    if kind == "wide":      # magnitudes over ten octaves of ten, row by row
+        x = x * torch.logspace(-6, 4, shape[-2], base=10.0)[:, None]
+    elif kind == "tiny":
+        x = x * 1e-6
+    elif kind == "ties":    # a coarse grid: many values halfway between two codes
+        x = torch.round(x * 4) / 4
+    elif kind == "outlier":
+        x = torch.where(torch.rand(shape, generator=g) < 0.01, x * 50, x)
+    x = x.to(dtype)
+    return x.clamp(-60000, 60000) if dtype == torch.float16 else x
+
+
+KINDS = ["normal", "wide", "tiny", "ties", "outlier"]
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_mx_quant_random(cuda, seed):
+    from mindiesd.layers.quant import mx_quantize
+    from oracle import quant as oq
+    r = random.Random(300 + seed)
+    dtype, kind = r.choice([torch.bfloat16, torch.float16]), r.choice(KINDS)
+    m, k = r.choice([1, 5, 31, 32, 33, 127, 128, 129, 300, 1000]), r.choice([32, 64, 128, 256, 320, 512, 1024])
+    x = _values((m, k), seed, dtype, kind)
+    q, e = mx_quantize(x.to(cuda))
+    codes, e8 = oq.mx_quant(x)
+    got = q.view(torch.uint8).cpu()
+    assert torch.equal(e.view(torch.uint8).cpu(), e8), (m, k, dtype, kind)
+    assert torch.equal(got & 0x7f, codes & 0x7f), (m, k, dtype, kind)
+    assert torch.equal((got >> 7)[codes & 0x7f != 0], (codes >> 7)[codes & 0x7f != 0])  # the sign of a zero is free
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_block_quant_random(cuda, seed):
+    from mindiesd.layers.quant.block_quant import _block_quant
+    from oracle import quant as oq
+    r = random.Random(400 + seed)
+    dtype, kind = r.choice([torch.bfloat16, torch.float16]), r.choice(KINDS)
+    s, n = r.choice([1, 100, 127, 128, 129, 256, 300, 1000]), r.choice([1, 2, 3])
+    layout, pow2, pre = r.choice(["BNSD", "BSND"]), r.random() < 0.5, r.choice([1.0, 1.0, 0.127, 3.5])
+    x = _values((1, n, s, 128), seed, dtype, kind)
+    xd = x.to(cuda) if layout == "BNSD" else x.transpose(1, 2).contiguous().to(cuda)
+    c, sc = _block_quant(xd, 128, layout, pre, pow2)
+    wc, ws = oq.dynamic_block_quant(x, 128, 128, pre, pow2)
+    got = c.cpu().view(torch.uint8)
+    assert torch.equal(sc.cpu(), ws[..., 0]), (n, s, dtype, kind, layout, pow2, pre)
+    zero = ((got & 0x7f) == 0) & ((wc & 0x7f) == 0)
+    assert bool(((got == wc) | zero).all()), (n, s, dtype, kind, layout, pow2, pre)
