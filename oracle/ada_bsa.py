@@ -163,10 +163,14 @@ def sparse_estimate(query, key, blocksize=128, stride=8, threshold=0.5, force_sp
     return mask
 
 
-def ada_block_sparse_attention(query, key, value, smask, causal=False, blocksize=128):
+def ada_block_sparse_attention(query, key, value, smask, causal=False, blocksize=128, rules="numpy"):
     """test_adablocksparseattention.py:35-87: every query block attends to the keys of the blocks its mask row
     selects; with ``causal`` the upper triangle of the last ``t`` gathered keys (``t`` = rows of the query
-    block) gets -10000 added, i.e. the last selected block is taken to be the diagonal block."""
+    block) gets -10000 added, i.e. the last selected block is taken to be the diagonal block.
+    ``rules="kernel"``: the reference kernel applies that triangle only when the last selected block IS the
+    diagonal block (``isLastBlockCausalDiag``, ada_block_sparse_attention_s1s2_bns1_x910.h:245-259, :512-514);
+    the two statements agree on every mask whose rows end with their diagonal block (what the estimate
+    produces with ``keep_recent``)."""
     bs, nq, seq, dim = query.shape
     gqa = nq // key.shape[1]
     out = torch.zeros(bs, nq, seq, dim, dtype=torch.float32)
@@ -182,7 +186,7 @@ def ada_block_sparse_attention(query, key, value, smask, causal=False, blocksize
                 if k.shape[0] == 0:
                     continue
                 p = qf[bi, ni, start:end] @ k.T / np.sqrt(dim)
-                if causal:
+                if causal and (rules == "numpy" or np.flatnonzero(sm[bi, ni, s1, :nb])[-1] == s1):
                     t = end - start
                     p[:, -t:] += np.triu(np.ones((t, t)), k=1) * (-10000.0)
                 p = p - p.max(axis=-1, keepdims=True)

@@ -192,6 +192,28 @@ def test_ada_block_sparse_attention_vs_oracle(cuda, causal, layout):
         assert not out[0, 3, 512:640].any()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_ada_attention_causal_rows_without_their_diagonal_block(cuda, seed):
+    """Random masks inside the lower triangle whose rows need not end with their diagonal block.  The reference
+    kernel masks inside a block only when the row's last selected block is the diagonal one
+    (ada_block_sparse_attention_s1s2_bns1_x910.h:512-514); its numpy test statement masks the last selected block
+    whatever it is.  The build tests key <= query by token index, which is the kernel's rule on such masks."""
+    import mindiesd  # noqa: F401
+    g = torch.Generator().manual_seed(seed)
+    s = (500, 769, 1100, 1537, 256, 130)[seed]
+    nb = (s + 127) // 128
+    q, k, v = _rand((2, 4, s, 128), seed, torch.bfloat16), _rand((2, 2, s, 128), seed + 1, torch.bfloat16), _rand((2, 2, s, 128), seed + 2, torch.bfloat16)
+    m = (torch.rand(2, 4, nb, nb, generator=g) > 0.5) & torch.ones(nb, nb).tril().bool()
+    smask = torch.zeros(2, 4, nb, 32, dtype=torch.int8)
+    smask[..., :nb] = m.to(torch.int8)
+    want = oab.ada_block_sparse_attention(q, k, v, m.numpy(), causal=True, rules="kernel")
+    out = torch.ops.mindiesd.ada_block_sparse_attention(
+        q.to(cuda), k.to(cuda), v.to(cuda), smask.to(cuda), m.sum(-1).to(torch.int32).to(cuda), input_layout="BNSD",
+        sparse_size=128, num_heads=4, num_key_value_heads=2, scale_value=128 ** -0.5, causal=True).cpu()
+    eb, ok, mx = ref_compare(want, out, 2.0 ** -6)
+    assert ok, (eb, mx)
+
+
 def test_sparse_attention_front_door_ada_bsa(cuda):
     from mindiesd import sparse_attention
     from mindiesd.layers.flash_attn.sparse_flash_attn_ada_bsa import get_estimate_mask

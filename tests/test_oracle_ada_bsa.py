@@ -181,3 +181,28 @@ def test_causal_estimate_kernel_rules_invariants():
     assert np.array_equal(full, np.tril(np.ones_like(full)))
     n = oab.sparse_estimate(q, k, threshold=0.7, force_sparse=1.0, rules="kernel")[0, 0]
     assert n[:, 0].all() and n[:, -1].all()
+
+
+def test_ada_attention_causal_rules_agree_when_rows_end_with_their_diagonal_block():
+    """The reference's numpy statement (triangle on the last selected block) and its kernel (triangle only when that
+    block is the diagonal one) are the same function on masks whose rows end with the diagonal block, and differ
+    where a row ends below it."""
+    import numpy as np
+    import torch
+    from oracle import ada_bsa as oab
+    g = torch.Generator().manual_seed(0)
+    s, nb = 300, 3
+    q, k, v = (torch.randn((1, 1, s, 128), generator=g).to(torch.bfloat16) for _ in range(3))
+    m = np.tril(np.ones((nb, nb), dtype=bool))[None, None]
+    a = oab.ada_block_sparse_attention(q, k, v, m, causal=True, rules="numpy")
+    b = oab.ada_block_sparse_attention(q, k, v, m, causal=True, rules="kernel")
+    assert torch.equal(a, b)
+    m2 = m.copy()
+    m2[0, 0, 2, 2] = False          # the last row ends with block 1, below its diagonal block
+    a = oab.ada_block_sparse_attention(q, k, v, m2, causal=True, rules="numpy")
+    b = oab.ada_block_sparse_attention(q, k, v, m2, causal=True, rules="kernel")
+    assert torch.equal(a[:, :, :256], b[:, :, :256]) and not torch.equal(a[:, :, 256:], b[:, :, 256:])
+    # kernel rule, row without its diagonal block: plain attention over the selected blocks
+    sel = torch.cat([k[0, 0, :256]]), torch.cat([v[0, 0, :256]])
+    p = torch.softmax(q[0, 0, 256:].float() @ sel[0].float().T / 128 ** 0.5, dim=-1) @ sel[1].float()
+    assert torch.allclose(b[0, 0, 256:], p, atol=1e-5)
