@@ -411,9 +411,12 @@ def block_sparse_attention_varlen(query, key, value, block_sparse_mask, scale, s
         raise ParametersInvalid("Inconsistent query/key/value head counts or dtypes.")
     sq, skv = max(lq), max(lk)
     qb, kb = (sq + BLOCK - 1) // BLOCK, (skv + BLOCK - 1) // BLOCK
-    if block_sparse_mask.dim() != 4 or tuple(block_sparse_mask.shape) != (b, n, qb, kb):
-        raise ParametersInvalid(f"block_sparse_mask must be [B, N, {qb}, {kb}], but got {tuple(block_sparse_mask.shape)}.")
-    idx, cnt = mask_to_lists(block_sparse_mask)
+    # a mask sized for the padded tensors (more block rows / columns than the longest sequence needs) is cut down
+    if (block_sparse_mask.dim() != 4 or tuple(block_sparse_mask.shape[:2]) != (b, n) or block_sparse_mask.shape[2] < qb
+            or block_sparse_mask.shape[3] < kb):
+        raise ParametersInvalid(f"block_sparse_mask must be [B, N, >= {qb}, >= {kb}] = [{b}, {n}, ...], "
+                                f"but got {tuple(block_sparse_mask.shape)}.")
+    idx, cnt = mask_to_lists(block_sparse_mask[:, :, :qb, :kb])
     meta = torch.tensor([[starts_q[i], lq[i], starts_k[i], lk[i]] for i in range(b)], dtype=torch.int32).to(q.device)
     o_str = (0, out.stride(1), out.stride(0)) if layout == "TND" else _strides_bns(out, layout)
     with torch.cuda.device(q.device):

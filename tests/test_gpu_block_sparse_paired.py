@@ -222,3 +222,14 @@ def test_block_sparse_op_with_per_batch_lengths(cuda):
     with pytest.raises(RuntimeError):
         torch.ops.mindiesd.block_sparse_attention(q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda),
                                                   actual_seq_lengths=[901, 5], actual_seq_lengths_kv=lens_kv)
+    # every sequence shorter than the tensors: a mask sized for the tensors is accepted, its leading blocks are used
+    lens_q, lens_kv = [300, 129], [257, 640]
+    out2, _ = torch.ops.mindiesd.block_sparse_attention(
+        q.to(cuda), k.to(cuda), v.to(cuda), m.to(torch.int8).to(cuda), scale_value=128 ** -0.5,
+        actual_seq_lengths=lens_q, actual_seq_lengths_kv=lens_kv, softmax_lse_flag=1)
+    for b in range(2):
+        lq, lk = lens_q[b], lens_kv[b]
+        qb, kb = (lq + 127) // 128, (lk + 127) // 128
+        want = oa.block_sparse_attention(q[b:b + 1, :, :lq], k[b:b + 1, :, :lk], v[b:b + 1, :, :lk], m[b:b + 1, :, :qb, :kb].numpy())
+        assert oa.ref_compare(want, out2[b:b + 1, :, :lq].cpu(), 2.0 ** -6)[1]
+        assert not out2[b, :, lq:].any()
