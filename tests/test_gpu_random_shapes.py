@@ -143,3 +143,52 @@ def test_block_quant_random(cuda, seed):
     assert torch.equal(sc.cpu(), ws[..., 0]), (n, s, dtype, kind, layout, pow2, pre)
     zero = ((got & 0x7f) == 0) & ((wc & 0x7f) == 0)
     assert bool(((got == wc) | zero).all()), (n, s, dtype, kind, layout, pow2, pre)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_varlen_random_sequences(cuda, seed):
+    import mindiesd
+    from oracle.attention import attention_varlen
+    r = random.Random(500 + seed)
+    nseq, (n, nkv), causal, d = r.randint(1, 6), _heads(r), r.random() < 0.5, r.choice([128, 128, 64])
+    lens_q = [r.choice([0, 1, 7, 64, 100, 129, 300, 513]) for _ in range(nseq)]
+    lens_k = [r.choice([1, 5, 64, 77, 128, 200, 257, 640]) for _ in range(nseq)]
+    if sum(lens_q) == 0:
+        lens_q[0] = 5
+    cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+    cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+    q, k, v = (_rnd((sum(lens_q), n, d), seed, torch.bfloat16), _rnd((sum(lens_k), nkv, d), seed + 1, torch.bfloat16),
+               _rnd((sum(lens_k), nkv, d), seed + 2, torch.bfloat16))
+    on_device = r.random() < 0.5   # the cumulative lengths may live on either side
+    out = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu_q.to(cuda) if on_device else cu_q,
+                                            cu_k.to(cuda) if on_device else cu_k, causal=causal).cpu()
+    want = attention_varlen(q, k, v, cu_q, cu_k, d ** -0.5, causal)
+    assert not torch.isnan(out.float()).any()
+    # short sequences: few keys per row, see test_masked_or_causal_random_shape for the bound
+    assert (out.float() - want.float()).abs().max().item() <= 5e-2, (lens_q, lens_k, n, nkv, d, causal)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_ada_attention_random_mask(cuda, seed):
+    import mindiesd  # noqa: F401
+    from oracle import ada_bsa as oab
+    r = random.Random(600 + seed)
+    s, (n, nkv), b = r.choice([130, 256, 500, 769, 1100, 1537]), _heads(r), r.choice([1, 2])
+    causal, layout, dtype = r.random() < 0.5, r.choice(["BNSD", "BSND"]), r.choice([torch.bfloat16, torch.float16])
+    nb = (s + 127) // 128
+    q, k, v = _rnd((b, n, s, 128), seed, dtype), _rnd((b, nkv, s, 128), seed + 1, dtype), _rnd((b, nkv, s, 128), seed + 2, dtype)
+    g = torch.Generator().manual_seed(seed)
+    m = torch.rand(b, n, nb, nb, generator=g) > r.choice([0.2, 0.5, 0.8])
+    if causal:
+        m &= torch.ones(nb, nb).tril().bool()
+    smask = torch.zeros(b, n, nb, (nb + 31) // 32 * 32, dtype=torch.int8)
+    smask[..., :nb] = m.to(torch.int8)
+    want = oab.ada_block_sparse_attention(q, k, v, m.numpy(), causal=causal, rules="kernel")
+    args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = torch.ops.mindiesd.ada_block_sparse_attention(
+        *(t.to(cuda) for t in args), smask.to(cuda), m.sum(-1).to(torch.int32).to(cuda), input_layout=layout,
+        sparse_size=128, num_heads=n, num_key_value_heads=nkv, scale_value=128 ** -0.5, causal=causal).cpu()
+    out = out if layout == "BNSD" else out.transpose(1, 2)
+    assert not torch.isnan(out.float()).any()
+    eb, ok, mx = oa.ref_compare(want, out, 2.0 ** -6)
+    assert ok, (eb, mx, b, n, nkv, s, causal, layout, dtype)
