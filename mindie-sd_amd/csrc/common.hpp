@@ -156,11 +156,6 @@ __device__ __forceinline__ float quarter_max(float v) {
   row_swap(v, e, o);
   return half_max(fmaxf(e, o));
 }
-__device__ __forceinline__ float quarter_sum(float v) {
-  float e, o;
-  row_swap(v, e, o);
-  return half_sum(e + o);
-}
 
 // Rescale of one 16-query column block of fa_fwd16_kernel when its reference maximum moves: l *= alpha, the seed and
 // the 8 score blocks -= delta, the 8 output blocks *= alpha - 69 registers updated in place by three asm blocks, each
