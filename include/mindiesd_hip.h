@@ -264,14 +264,20 @@ int mindiesd_fp8_v_quant_static(const void* v, void* v8t, float* v_scale, int dt
 /* FP8 flash attention on operands produced by the two functions above (Q/K with block_size 128).
  * Replaces torch_npu.npu_fused_infer_attention_score_v2 with per-block dequantisation scales as
  * called by FP8RotateQuantFA.forward (mindiesd/quantization/layer.py:304-316).
- * log2_domain != 0: q_scale and k_scale hold powers of two and the query was quantised with
- * prescale = softmax scale * log2(e) (pow2_scale quantisation above); the scales are then applied by the matrix
- * instruction's exponent operands and `scale` is not used.  Same result up to the quantisation recipe, about
- * 12 % faster. */
+ * flags (bits, 0 = the default):
+ *   MSD_FP8_LOG2_DOMAIN  q_scale and k_scale hold powers of two and the query was quantised with
+ *                        prescale = softmax scale * log2(e) (pow2_scale quantisation above); the scales are then
+ *                        applied by the matrix instruction's exponent operands and `scale` is not used.
+ *   MSD_FP8_P_EXP2       the probabilities of a tile are 2^(score - reference) by the exponential instruction, rounded
+ *                        to E4M3 (the older, slower rule).  Default: the E4M3 code of a probability is computed
+ *                        directly as round(8 * (score - reference) + const), i.e. the exponential with its mantissa
+ *                        interpolated linearly between powers of two; the denominator is summed from the same codes. */
+#define MSD_FP8_LOG2_DOMAIN 1
+#define MSD_FP8_P_EXP2 2
 int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
                                const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
                                int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,
-                               int log2_domain, hipStream_t stream);
+                               int flags, hipStream_t stream);
 
 /* ---- MXFP8 linear layer --------------------------------------------------------------------------------
  * x [M][K] 16-bit (row stride x_stride elements) -> q [M][K] E4M3 + e8m0 [M][K/32]

@@ -348,10 +348,25 @@ struct Fp8Params {
   float scale_log2;  // softmax scale * log2(e)
 };
 
-// P is scaled by 2^kPShift before the E4M3 conversion; with the lazy-maximum threshold kTau8 the
-// largest value is 2^(kTau8 + kPShift) = 256 <= 448 and values down to 2^-13 survive as subnormals.
+// Two rules for the E4M3 probabilities of a tile (x = score - reference maximum, in log2 units):
+//  * PL = false ("exp2"): P = 2^(x + kPShift) by v_exp_f32, rounded by v_cvt_pk_fp8_f32.  With the lazy-maximum
+//    threshold kTau8 the largest value is 2^(kTau8 + kPShift) = 256 <= 448 and values down to 2^-13 survive as
+//    subnormals.
+//  * PL = true ("linear", the default): the E4M3 CODE itself is computed, code = rne(8 * (x + kShiftL + 7)) saturated
+//    to [0, 255] by v_cvt_pk_u8_f32.  An E4M3 code read as an integer is 8 * (exponent + 7) + mantissa eighths, so
+//    this is 2^floor(x') * (1 + frac(x')) with frac rounded to eighths (x' = x + kShiftL): the exponential with its
+//    mantissa interpolated linearly between powers of two, at most 6 % above 2^x'.  The denominator is summed from
+//    the same codes, so the common factor cancels; what is left is a relative error of 3 % rms per probability, the
+//    size of the E4M3 rounding itself.  One multiply-add and one conversion per score replace multiply-add,
+//    exponential and half an E4M3 pack (the two quarter-rate instructions of the other rule).  Codes below 8
+//    (x' < -6) are the format's subnormals, where the linear rule falls off faster than 2^x'; the shift is therefore
+//    as large as E4M3 allows (2^(kTauL + kShiftL) = 2^8.75 = 431 <= 448, code 126) so that only probabilities below
+//    2^-13.75 of the reference maximum are affected, and the threshold for moving the reference is 2^kTauL.
 constexpr float kTau8 = 4.0f;
 constexpr float kPShift = 4.0f;
+constexpr float kTauL = 1.0f;
+constexpr float kShiftL = 7.75f;
+constexpr float kSeedL = 8.0f * (kShiftL + 7.0f);  // the code of x = 0
 
 // 8 waves x 32 query rows, 128-key tiles, K tile [key][128 B] and V^T tile [channel][128 B] in LDS
 // (16 KiB each, double buffered); 16-byte chunk c of row r is stored at chunk c ^ ((r >> 1) & 7).
@@ -359,7 +374,9 @@ constexpr float kPShift = 4.0f;
 // times log2(e).  The two scales then go into the exponent operands of the scaled matrix instruction and the
 // score accumulators are seeded with kPShift - m, so the matrix core delivers s - m + kPShift and the softmax is
 // exp2 and rounding alone (no multiply-add per score).
-template <int DT, bool P2>
+// (launch bounds: 8 waves per workgroup, at least 2 waves per SIMD = the one workgroup a CU holds with 96 KiB of LDS;
+// the register budget is 256 per lane)
+template <int DT, bool P2, bool PL>
 __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
@@ -400,7 +417,12 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   const int qblk = min((q0 + wave * 32) >> 7, qblocks - 1);
   const float q_sc_raw = p.q_scale[(long long)bn * qblocks + qblk];
   const float q_sc = q_sc_raw * p.scale_log2;
-  const int q_exp = (int)((__builtin_bit_cast(unsigned, q_sc_raw) >> 23) & 0xffu);  // E8M0 code of a power of two
+  // E8M0 code of a power of two; the factor 8 of the linear code rule rides on it
+  const int q_exp = (int)((__builtin_bit_cast(unsigned, q_sc_raw) >> 23) & 0xffu) + (PL ? 3 : 0);
+  // seed of the score accumulators at reference 0, lazy threshold and units per log2 step in the accumulator's domain
+  constexpr float kSeed = PL ? kSeedL : kPShift;
+  constexpr float kUnit = PL ? 8.0f : 1.0f;
+  constexpr float kTau = PL ? kTauL : kTau8;
   // read through the constant address space: a scalar load, which does not queue behind the tile requests
   typedef const __attribute__((address_space(4))) float* ConstF;
   const ConstF k_sc = (ConstF)(uintptr_t)(p.k_scale + (long long)bn * kblocks);
@@ -411,9 +433,9 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
   float m_run = P2 ? 0.f : -INFINITY;
-  f32x16_t negm;  // P2: kPShift - m_run in every slot, the seed of the score accumulators
+  f32x16_t negm;  // P2: kSeed - kUnit * m_run in every slot, the seed of the score accumulators
 #pragma unroll
-  for (int r = 0; r < 16; ++r) negm[r] = kPShift;
+  for (int r = 0; r < 16; ++r) negm[r] = kSeed;
   bool first = true;
 
   // ---- LDS-DMA staging: one instruction = 8 rows x 128 bytes ----------------------------------------------------
@@ -518,10 +540,10 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
     i32x8_t pf[2];
     if (P2) {
-      // sacc = s - m_run + kPShift; the reference maximum moves when a row exceeds it by more than kTau8
+      // sacc = kUnit * (s - m_run) + kSeed; the reference maximum moves when a row exceeds it by more than kTau
       // (tested on the lanes' own parts: one of them exceeds the threshold iff a row maximum does)
-      mx -= kPShift;
-      if (first || __builtin_amdgcn_ballot_w64(mx > kTau8) != 0) {
+      mx = (mx - kSeed) * (1.0f / kUnit);
+      if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
         mx = half_max(mx);
         float delta = first ? mx : fmaxf(mx, 0.f);
         delta = (delta == -INFINITY) ? 0.f : delta;
@@ -529,11 +551,11 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
         const float alpha = first ? 1.f : fast_exp2(-delta);
         m_run += delta;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) negm[r] = kPShift - m_run;
+        for (int r = 0; r < 16; ++r) negm[r] = kSeed - kUnit * m_run;
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sacc[kb][r] -= delta;
+          for (int r = 0; r < 16; ++r) sacc[kb][r] -= kUnit * delta;
 #pragma unroll
         for (int r = 0; r < 16; ++r) lacc[r] *= alpha;
 #pragma unroll
@@ -544,7 +566,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
       first = false;
     } else {
     mx *= c;
-    if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau8) != 0) {
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + kTau) != 0) {
       mx = half_max(mx);
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2(m_run - (m_new == -INFINITY ? 0.f : m_new));
@@ -558,13 +580,25 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     }
     }  // !P2
     const float mc = P2 ? 0.f : (m_run == -INFINITY ? 0.f : m_run) - kPShift;
+    // linear rule: code = c8 * raw score + off8 with off8 = kSeedL - 8 * reference
+    const float c8 = c * 8.0f;
+    const float off8 = __builtin_fmaf(-8.0f, m_run == -INFINITY ? 0.f : m_run, kSeedL);
     // probabilities of keys 64 * kk .. + 64 of the tile, rounded to E4M3 and packed as the B operand
     auto exp_pack = [&](const int kk) {
 #pragma unroll
       for (int kb = 2 * kk; kb < 2 * kk + 2; ++kb) {
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-          if (P2)
+          if (PL) {
+            unsigned w;
+            asm volatile("" : "=v"(w));  // any register content: all four bytes are overwritten
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float y = P2 ? sacc[kb][4 * g4 + j] : __builtin_fmaf(sacc[kb][4 * g4 + j], c8, off8);
+              w = __builtin_amdgcn_cvt_pk_u8_f32(y, j, w);
+            }
+            pf[kk][(kb & 1) * 4 + g4] = (int)w;
+          } else if (P2)
             pf[kk][(kb & 1) * 4 + g4] =
                 pack4_e4m3_noclamp(fast_exp2(sacc[kb][4 * g4]), fast_exp2(sacc[kb][4 * g4 + 1]),
                                    fast_exp2(sacc[kb][4 * g4 + 2]), fast_exp2(sacc[kb][4 * g4 + 3]));
@@ -594,7 +628,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     __builtin_amdgcn_sched_barrier(0);
     pv(0);
     exp_pack(1);
-    constexpr int kValuPerMfma = P2 ? 10 : 16;
+    constexpr int kValuPerMfma = PL ? (P2 ? 8 : 14) : (P2 ? 10 : 16);
     __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
@@ -648,6 +682,17 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
     if (qr < p.Sq) *(i32x4_t*)(og + (long long)qr * p.o_ss + c16 * 8) = i32x4_t{lo[0], lo[1], hi[0], hi[1]};
   }
 #endif
+}
+
+// grid = one workgroup per 256 query rows of a (batch, head), rounded up to a multiple of 8
+template <int DT, bool P2, bool PL>
+int fp8_fa_launch(const Fp8Params& p, int grid, hipStream_t stream) {
+  constexpr int kLds = 3 * 32768;  // 3 stages x 32 KiB; the output staging (66 KiB) reuses them
+  auto kern = fp8_fa_fwd_kernel<DT, P2, PL>;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+    return MSD_ERR_LAUNCH;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
 }  // namespace msd
@@ -780,11 +825,12 @@ int mindiesd_fp8_v_quant_static(const void* v, void* v8t, float* v_scale, int dt
 int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
                                const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
                                int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,
-                               int log2_domain, hipStream_t stream) {
+                               int flags, hipStream_t stream) {
   if (!q8 || !k8 || !v8t || !q_scale || !k_scale || !v_scale || !out) return MSD_ERR_BAD_ARG;
   if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return MSD_ERR_BAD_ARG;
   if (D != 128 || !(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
   if (out_dtype != MSD_DTYPE_BF16 && out_dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
+  if (flags & ~(MSD_FP8_LOG2_DOMAIN | MSD_FP8_P_EXP2)) return MSD_ERR_BAD_ARG;
   if (((uintptr_t)q8 | (uintptr_t)k8 | (uintptr_t)v8t | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
   if ((o_sb | o_sn | o_ss) & 7) return MSD_ERR_BAD_ARG;
   const int S128 = (Skv + 127) / 128 * 128;
@@ -795,36 +841,19 @@ int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, 
   p.o = out; p.o_sb = o_sb; p.o_sn = o_sn; p.o_ss = o_ss;
   p.B = B; p.N = N; p.Sq = Sq; p.Skv = Skv; p.S128 = S128;
   p.scale_log2 = scale * 1.4426950408889634f;
-  constexpr int kLds = 3 * 32768;  // 3 stages x 32 KiB; the output staging (66 KiB) reuses them
   const int q_tiles = (Sq + 255) / 256;
   const int total = B * N * q_tiles;
   const int grid = (total + 7) / 8 * 8;
-  if (log2_domain) {
-    if (out_dtype == MSD_DTYPE_BF16) {
-      auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16, true>;
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-        return MSD_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
-    } else {
-      auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16, true>;
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-        return MSD_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
-    }
-    return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
-  }
-  if (out_dtype == MSD_DTYPE_BF16) {
-    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_BF16, false>;
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-      return MSD_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
-  } else {
-    auto kern = fp8_fa_fwd_kernel<MSD_DTYPE_F16, false>;
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-      return MSD_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, p);
-  }
-  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+  const bool bf = out_dtype == MSD_DTYPE_BF16;
+  const bool p2 = (flags & MSD_FP8_LOG2_DOMAIN) != 0, pl = (flags & MSD_FP8_P_EXP2) == 0;
+  if (p2 && pl) return bf ? fp8_fa_launch<MSD_DTYPE_BF16, true, true>(p, grid, stream)
+                          : fp8_fa_launch<MSD_DTYPE_F16, true, true>(p, grid, stream);
+  if (p2) return bf ? fp8_fa_launch<MSD_DTYPE_BF16, true, false>(p, grid, stream)
+                    : fp8_fa_launch<MSD_DTYPE_F16, true, false>(p, grid, stream);
+  if (pl) return bf ? fp8_fa_launch<MSD_DTYPE_BF16, false, true>(p, grid, stream)
+                    : fp8_fa_launch<MSD_DTYPE_F16, false, true>(p, grid, stream);
+  return bf ? fp8_fa_launch<MSD_DTYPE_BF16, false, false>(p, grid, stream)
+            : fp8_fa_launch<MSD_DTYPE_F16, false, false>(p, grid, stream);
 }
 
 }  // extern "C"

@@ -47,7 +47,7 @@ register_ops.define_op(
 register_ops.define_op(
     "fp8_attention_fwd",
     "(Tensor query, Tensor key, Tensor value, float scale_value=1.0, str input_layout='BNSD', Tensor? q_rot=None, "
-    "Tensor? k_rot=None, str recipe='amax') -> Tensor")
+    "Tensor? k_rot=None, str recipe='amax', str p_rule='linear') -> Tensor")
 register_ops.define_op(
     "mxfp8_gemm_swiglu",
     "(Tensor x, Tensor weight, Tensor weight_scale, Tensor? bias=None, bool swiglu=True) -> Tensor")
@@ -293,7 +293,7 @@ def _sparse_block_estimate_impl(query, key, actual_seq_lengths=None, actual_seq_
 @register_ops.register_mindie_fake_op("sparse_block_estimate")
 def sparse_block_estimate_fake(query, key, actual_seq_lengths=None, actual_seq_lengths_kv=None, input_layout="BNSD",
                                stride=8, sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0,
-                               threshold=1.0, causal=True, keep_sink=True, keep_recent=True, row_sparse=1.0):
+                               threshold=1.0, causal=False, keep_sink=True, keep_recent=True, row_sparse=1.0):
     b, nq, s = (query.shape[0], query.shape[1], query.shape[2]) if input_layout == "BNSD" else \
         (query.shape[0], query.shape[2], query.shape[1])
     nb = (s + sparse_size - 1) // sparse_size
@@ -304,7 +304,7 @@ def sparse_block_estimate_fake(query, key, actual_seq_lengths=None, actual_seq_l
 def sparse_block_estimate(query, key, actual_seq_lengths: Optional[List[int]] = None,
                           actual_seq_lengths_kv: Optional[List[int]] = None, input_layout: str = "BNSD",
                           stride: int = 8, sparse_size: int = 128, num_heads: int = 1, num_key_value_heads: int = 1,
-                          scale_value: float = 1.0, threshold: float = 1.0, causal: bool = True,
+                          scale_value: float = 1.0, threshold: float = 1.0, causal: bool = False,
                           keep_sink: bool = True, keep_recent: bool = True,
                           row_sparse: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
     return torch.ops.mindiesd.sparse_block_estimate(
@@ -329,8 +329,8 @@ def _ada_block_sparse_attention_impl(query, key, value, sparse_mask, sparse_coun
 
 @register_ops.register_mindie_fake_op("ada_block_sparse_attention")
 def ada_block_sparse_attention_fake(query, key, value, sparse_mask, sparse_count_table, input_layout="BNSD",
-                                    sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0, causal=True,
-                                    inner_precise=1, pre_tokens=214748647, next_tokens=0, actual_seq_lengths=None,
+                                    sparse_size=128, num_heads=1, num_key_value_heads=1, scale_value=1.0, causal=False,
+                                    inner_precise=1, pre_tokens=214748647, next_tokens=214748647, actual_seq_lengths=None,
                                     actual_seq_lengths_kv=None):
     return torch.empty_like(query)
 
@@ -366,14 +366,14 @@ def _fa_block_quant_fake(x, block_size=128, input_layout="BNSD"):
 
 @register_ops.register_device_impl("fp8_attention_fwd")
 def _fp8_attention_fwd_impl(query, key, value, scale_value=1.0, input_layout="BNSD", q_rot=None, k_rot=None,
-                            recipe="amax"):
+                            recipe="amax", p_rule="linear"):
     from .quant.fp8_attention import fp8_attention_forward
-    return fp8_attention_forward(query, key, value, scale_value, input_layout, q_rot, k_rot, recipe)
+    return fp8_attention_forward(query, key, value, scale_value, input_layout, q_rot, k_rot, recipe, p_rule)
 
 
 @register_ops.register_mindie_fake_op("fp8_attention_fwd")
 def _fp8_attention_fwd_fake(query, key, value, scale_value=1.0, input_layout="BNSD", q_rot=None, k_rot=None,
-                            recipe="amax"):
+                            recipe="amax", p_rule="linear"):
     return torch.empty_like(query)
 
 

@@ -105,7 +105,7 @@ def avgpool(input_tensor, pool_size=128, input_layout="BNSD"):
 # ------------------------------------------------------------------------------------------------
 # rf_v2.py:137-289
 # ------------------------------------------------------------------------------------------------
-def rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k=None, input_layout="BNSD"):
+def rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k, input_layout):
     """8x8-window token order (all frames if h and w are multiples of 8, else frames 1.. with the
     remainder rows/columns appended per frame).  Only ``latent_shape_q`` is used, as in the reference."""
     _check_layout(input_layout)
@@ -117,7 +117,8 @@ def rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k=None, input_
     return out
 
 
-def inv_rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k=None, input_layout="BNSD"):
+def inv_rearrange_with_remaining(tensor, latent_shape_q, latent_shape_k, input_layout):
+    """Back from the 8x8-window order to T-H-W order (rf_v2.py:199-289)."""
     _check_layout(input_layout)
     _check_gpu16(tensor, "tensor")
     x = _aligned(tensor)
@@ -175,6 +176,20 @@ def do_tensor_inv_rearrange(tensor, text_len, latent_shape_q, latent_shape_k, in
     out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     _run_rearrange([x], [out], None, input_layout, grid, text_len, 1)
     return out
+
+
+def _bsa_inv_rearrange(out, tq, hq, wq, input_layout="BSND"):
+    """The rf_v3 spelling of the inverse permutation without text tokens (rf_v3.py:22-97): the same token map as
+    ``inv_rearrange_with_remaining`` on the grid (tq, hq, wq)."""
+    return inv_rearrange_with_remaining(out, (tq, hq, wq), None, input_layout)
+
+
+def do_tensor_pooling(tensor, text_len):
+    """rf_v2.py:340-348 as written there: the tensor is cut at ``text_len`` along dim 1, both parts are pooled by
+    ``avgpool`` with its default layout (blocks of 128 along dim 2) and joined along dim 1, first part first."""
+    parts = [t for t in (tensor[:, :text_len], tensor[:, text_len:]) if t.shape[1] > 0]
+    pooled = [avgpool(t, pool_size=BLOCK) for t in parts]
+    return pooled[0] if len(pooled) == 1 else torch.concat(pooled, dim=1)
 
 
 # ------------------------------------------------------------------------------------------------

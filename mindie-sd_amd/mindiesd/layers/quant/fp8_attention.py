@@ -34,14 +34,21 @@ def quantize_v_per_channel(value, layout="BNSD"):
 
 
 LOG2E = 1.4426950408889634
+# flag bits of mindiesd_fp8_attention_fwd (include/mindiesd_hip.h)
+FLAG_LOG2_DOMAIN, FLAG_P_EXP2 = 1, 2
+P_RULES = ("linear", "exp2")
 
 
 def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_dtype=torch.bfloat16, layout="BNSD",
-                            log2_domain=False):
+                            log2_domain=False, p_rule="linear"):
     """Attention on already quantised operands (see ``quantize_v_per_channel`` and ``_block_quant``
     with block 128).  Output [B,N,S,128] ('BNSD') or [B,S,N,128] ('BSND') in ``out_dtype``.
     ``log2_domain``: the query was quantised with ``prescale = scale * log2(e)`` and both q and k with
-    power-of-two scales; ``scale`` is then not used."""
+    power-of-two scales; ``scale`` is then not used.
+    ``p_rule``: how a tile's probabilities become E4M3 - see ``fp8_attention_forward``."""
+    if p_rule not in P_RULES:
+        raise ParametersInvalid(f"p_rule must be one of {P_RULES}, but got {p_rule}.")
+    flags = (FLAG_LOG2_DOMAIN if log2_domain else 0) | (FLAG_P_EXP2 if p_rule == "exp2" else 0)
     b, n, sq, d = q8.shape
     skv = k8.shape[2]
     shape = (b, n, sq, d) if layout == "BNSD" else (b, sq, n, d)
@@ -50,12 +57,13 @@ def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_d
         rc = _native.lib().mindiesd_fp8_attention_fwd(
             q8.data_ptr(), k8.data_ptr(), v8t.data_ptr(), q_scale.data_ptr(), k_scale.data_ptr(), v_scale.data_ptr(),
             out.data_ptr(), _native.DTYPE_CODE[out_dtype], b, n, sq, skv, d, *_strides_bns(out, layout),
-            float(scale), int(bool(log2_domain)), _native.stream_ptr(q8.device))
+            float(scale), flags, _native.stream_ptr(q8.device))
     _native.check(rc, "mindiesd_fp8_attention_fwd")
     return out
 
 
-def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None, recipe="amax"):
+def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None, recipe="amax",
+                          p_rule="linear"):
     """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``.
     ``q_rot`` / ``k_rot`` ([128, 128]): query @ q_rot and key @ k_rot are formed inside the quantisation
     pass (the rotated tensors are never written).
@@ -65,7 +73,13 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=No
     operands and the softmax needs no multiply (about 4 % faster).  On inputs without outliers both give the same
     accuracy; with amax/448 the largest element of every block is encoded exactly (code 448), which 'pow2' gives
     up, and on inputs whose softmax is decided by a few outliers that costs accuracy (cosine 0.979 against 0.987
-    at 32760 tokens with 1 % of the elements scaled by 8)."""
+    at 32760 tokens with 1 % of the elements scaled by 8).
+    ``p_rule``: 'linear' (default) - the E4M3 code of a probability is computed directly as
+    round(8 * (score - reference) + const): the exponential with its mantissa interpolated linearly between powers of
+    two (at most 6 % above 2^x, 3 % rms after the common factor cancels against the denominator, which is summed
+    from the same codes) - one multiply-add and one conversion per score; 'exp2' - 2^(score - reference) by the
+    exponential instruction, rounded to E4M3 (slower: two quarter-rate instructions per score).  Both stay inside
+    the FP8 workload's tolerance (cosine >= 0.999 against the quantise -> dequantise path)."""
     for name, t in (("query", query), ("key", key), ("value", value)):
         if not isinstance(t, torch.Tensor) or t.dim() != 4:
             raise ParametersInvalid(f"The input {name} must be a 4-D torch.Tensor.")
@@ -88,4 +102,4 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=No
     k8, ks = (_block_quant(key, 128, layout, 1.0, p2) if k_rot is None
               else _rot_block_quant(key, k_rot, layout, 1.0, p2))
     v8t, vs = quantize_v_per_channel(value, layout)
-    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout, log2_domain=p2)
+    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout, log2_domain=p2, p_rule=p_rule)

@@ -113,7 +113,7 @@ def per_channel_quant(v):
     return torch.from_numpy(e4m3_encode(vf / sc[..., None, :])), torch.from_numpy(sc)
 
 
-def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False):
+def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False, p_rule="linear"):
     """FP8 attention of the Wan2.1-14B 480p workload, BNSD: Q and K quantised per (head, 128-token
     block) over all channels, V per (head, channel); bf16-typed output.
     ``requant_p=False``: the quantise -> dequantise path - everything is dequantised and run through plain
@@ -123,7 +123,12 @@ def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False):
     the reference is a running maximum per query row that is only moved when, in the row's group of 32 consecutive
     query rows, some row's tile maximum exceeds its reference by more than 2^4 (so P <= 256 < 448); the
     denominator is the sum of the ROUNDED probabilities, the numerator their product with the V codes; both are
-    rescaled by 2^(old - new reference) when the reference moves."""
+    rescaled by 2^(old - new reference) when the reference moves.  That is ``p_rule="exp2"``.
+    ``p_rule="linear"`` (the kernel's default): the E4M3 CODE of a probability is computed directly,
+    code = rne(8 * (score - reference) + 8 * (7.75 + 7)) saturated to [0, 255] - read back as E4M3 that is
+    2^floor(x') * (1 + frac(x')) with frac rounded to eighths, x' = score - reference + 7.75: the exponential with
+    its mantissa interpolated linearly between powers of two (code 8 e + m stands for 2^(e-7) (1 + m/8)); the reference
+    moves when a row of the group exceeds it by more than 2^1 (so the code stays <= 126 = 448)."""
     d = query.shape[-1]
     if scale is None:
         scale = d ** -0.5
@@ -138,7 +143,8 @@ def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False):
         kc, ks = dynamic_block_quant(key, 128, d)
     vc, vs = per_channel_quant(value)
     if requant_p:
-        return _fp8_attention_requant(qc, qs, kc, ks, vc, vs, np.float32(scale * 1.4426950408889634), pow2).to(query.dtype)
+        return _fp8_attention_requant(qc, qs, kc, ks, vc, vs, np.float32(scale * 1.4426950408889634), pow2,
+                                      p_rule).to(query.dtype)
     qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, 128, d)
     vd = torch.from_numpy(e4m3_decode(vc.numpy())) * vs[..., None, :]
     out = torch.empty(query.shape, dtype=torch.float32)
@@ -149,10 +155,21 @@ def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False):
 
 
 P_SHIFT, P_TAU, ROW_GROUP, KEY_TILE = np.float32(4.0), np.float32(4.0), 32, 128
+L_SHIFT, L_TAU = np.float32(7.75), np.float32(1.0)       # the linear code rule
+L_SEED = np.float32(8.0) * (L_SHIFT + np.float32(7.0))   # the code of score == reference (118)
 
 
-def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2):
+def linear_p_codes(y):
+    """E4M3 codes of the linear rule from y = 8 * (score - reference) + 118 (fp32): rne(y) saturated to [0, 255]
+    (what v_cvt_pk_u8_f32 does: ties to even, negative and NaN -> 0)."""
+    y = np.nan_to_num(np.asarray(y, np.float32), nan=0.0, posinf=255.0, neginf=0.0)
+    return np.clip(np.rint(y), 0, 255).astype(np.uint8)
+
+
+def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2, p_rule="linear"):
     """The tile loop behind ``fp8_attention(requant_p=True)`` on the quantised operands (codes + scales)."""
+    linear = p_rule == "linear"
+    tau = L_TAU if linear else P_TAU
     q8, k8, v8 = e4m3_decode(qc.numpy()), e4m3_decode(kc.numpy()), e4m3_decode(vc.numpy())
     qsn, ksn, vsn = qs.numpy()[..., 0], ks.numpy()[..., 0], vs.numpy()
     b, n, sq, d = q8.shape
@@ -174,7 +191,7 @@ def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2):
                     if pow2:  # the scales are powers of two (applied by the matrix instruction's exponents)
                         s = (raw * (qsc * ksn[bi, ni, t0 // 128])).astype(np.float32)
                         mx = s.max(axis=1) - m_run
-                        if first or (mx > P_TAU).any():
+                        if first or (mx > tau).any():
                             delta = mx if first else np.maximum(mx, np.float32(0))
                             # (first tile: sums and outputs are still zero, the factor is 1; 2^-delta may overflow)
                             alpha = np.ones_like(delta) if first else np.exp2(-delta).astype(np.float32)
@@ -185,14 +202,23 @@ def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2):
                         c = np.float32(np.float32(qsc * scale_log2) * ksn[bi, ni, t0 // 128])
                         s = (raw * c).astype(np.float32)
                         mx = s.max(axis=1)
-                        if (mx > m_run + P_TAU).any():
+                        if (mx > m_run + tau).any():
                             m_new = np.maximum(m_run, mx)
                             alpha = np.where(np.isinf(m_run), np.float32(0), np.exp2(m_run - m_new)).astype(np.float32)
                             m_run = m_new
                             l_run *= alpha
                             o_run *= alpha[:, None]
                     first = False
-                    p8 = e4m3_round(np.exp2(s - (m_run - P_SHIFT)[:, None]).astype(np.float32))
+                    if linear:
+                        # one multiply-add per score on the GPU: (8 c) raw + (118 - 8 reference), rounded once
+                        off8 = (np.float64(L_SEED) - 8.0 * m_run.astype(np.float64)).astype(np.float32)
+                        if pow2:  # the matrix instruction applies 8 x the two scales and starts from off8
+                            y = 8.0 * s.astype(np.float64) + off8[:, None]
+                        else:
+                            y = raw.astype(np.float64) * np.float64(np.float32(c * np.float32(8.0))) + off8[:, None]
+                        p8 = e4m3_decode(linear_p_codes(y.astype(np.float32)))
+                    else:
+                        p8 = e4m3_round(np.exp2(s - (m_run - P_SHIFT)[:, None]).astype(np.float32))
                     l_run += p8.sum(axis=1, dtype=np.float32)
                     o_run += p8 @ v8[bi, ni, t0:t1]
                 inv = np.where(l_run > 0, np.float32(1) / np.maximum(l_run, np.float32(1e-30)), np.float32(0))

@@ -93,19 +93,20 @@ def test_pow2_block_quant_bit_exact(cuda, prescale, layout):
         assert scale[0, 2, 0].item() == 4.0
 
 
+@pytest.mark.parametrize("p_rule", ["linear", "exp2"])
 @pytest.mark.parametrize("recipe", ["pow2", "amax"])
 @pytest.mark.parametrize("layout,s", [("BNSD", 1024), ("BNSD", 1100), ("BSND", 700)])
-def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
+def test_fp8_attention_vs_oracle(cuda, layout, s, recipe, p_rule):
     from mindiesd.layers.quant import fp8_attention_forward
     q, k, v = _outlier_inputs((1, 3, s, 128), seed=s)
     want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2")
     args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
-    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout, recipe=recipe).cpu()
+    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout, recipe=recipe, p_rule=p_rule).cpu()
     out = out if layout == "BNSD" else out.transpose(1, 2)
     assert out.dtype == torch.bfloat16 and out.shape == q.shape
     cos = cosine(out, want)
     err = (out.float() - want.float()).abs()
-    print(f"fp8 attention S={s} {layout}: cosine {cos:.6f}, max-abs {err.max():.4f}, mean-abs {err.mean():.5f}, "
+    print(f"fp8 attention S={s} {layout} {recipe} {p_rule}: cosine {cos:.6f}, max-abs {err.max():.4f}, mean-abs {err.mean():.5f}, "
           f"output rms {want.float().pow(2).mean().sqrt():.4f}")
     assert cos >= 0.999, f"cosine {cos}"
     # coarse guard against gross outliers: E4M3 probabilities carry 2^-4 relative noise per element
@@ -113,7 +114,7 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
     # against the oracle that re-quantises P the way the kernel does (same tiles, same reference rule, same
     # rounding): what is left is the summation order, the hardware's exp2 and a probability now and then landing on
     # the neighbouring E4M3 number
-    mirror = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True)
+    mirror = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True, p_rule=p_rule)
     cos_m = cosine(out, mirror)
     err_m = (out.float() - mirror.float()).abs()
     print(f"   vs the P-requantising oracle: cosine {cos_m:.7f}, max-abs {err_m.max():.5f}")
@@ -121,8 +122,9 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe):
     assert err_m.max() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("p_rule", ["linear", "exp2"])
 @pytest.mark.parametrize("recipe", ["pow2", "amax"])
-def test_fp8_attention_scores_far_below_zero(cuda, recipe):
+def test_fp8_attention_scores_far_below_zero(cuda, recipe, p_rule):
     """q near +8, k near -8: every score lies hundreds of units below zero, the first key tile moves the running
     maximum far down."""
     from mindiesd.layers.quant import fp8_attention_forward
@@ -131,8 +133,8 @@ def test_fp8_attention_scores_far_below_zero(cuda, recipe):
     q = (8.0 + 0.5 * torch.randn(shape, generator=g)).to(torch.bfloat16)
     k = (-8.0 + 0.5 * torch.randn(shape, generator=g)).to(torch.bfloat16)
     v = torch.randn(shape, generator=g).to(torch.bfloat16)
-    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True)
-    out = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), layout="BNSD", recipe=recipe).cpu()
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True, p_rule=p_rule)
+    out = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), layout="BNSD", recipe=recipe, p_rule=p_rule).cpu()
     assert not torch.isnan(out.float()).any()
     assert cosine(out, want) >= 0.999
 

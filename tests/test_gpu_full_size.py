@@ -111,16 +111,18 @@ def test_fp8_attention_wan14b_480p(cuda):
     # two query blocks of two heads against the quantise -> dequantise oracle (cosine >= 0.999)
     # (each recipe against the oracle of the same recipe)
     out_p2 = fp8_attention_forward(q, k, v, layout="BNSD", recipe="pow2")
+    out_ex = fp8_attention_forward(q, k, v, layout="BNSD", p_rule="exp2")
     for head in (0, 39):
         qs = q[:, head:head + 1, 128 * 100: 128 * 102].cpu()
-        for res, p2 in ((out, False), (out_p2, True)):
+        for res, p2, rule in ((out, False, "linear"), (out_p2, True, "linear"), (out_ex, False, "exp2")):
             want = oq.fp8_attention(qs, k[:, head:head + 1].cpu(), v[:, head:head + 1].cpu(), pow2=p2)
             got = res[:, head:head + 1, 128 * 100: 128 * 102].cpu()
             assert oa.cosine(got, want) >= 0.999, (p2, oa.cosine(got, want))
             # and tightly against the oracle that re-quantises P per tile the way the kernel does
-            mirror = oq.fp8_attention(qs, k[:, head:head + 1].cpu(), v[:, head:head + 1].cpu(), pow2=p2, requant_p=True)
+            mirror = oq.fp8_attention(qs, k[:, head:head + 1].cpu(), v[:, head:head + 1].cpu(), pow2=p2, requant_p=True,
+                                      p_rule=rule)
             assert oa.cosine(got, mirror) >= 0.99998, (p2, oa.cosine(got, mirror), oa.cosine(got, want))
-            print(f"fp8 full size head {head} pow2 {p2}: cosine vs plain oracle {oa.cosine(got, want):.7f}, vs P-requantising oracle {oa.cosine(got, mirror):.7f}", flush=True)
+            print(f"fp8 full size head {head} pow2 {p2} {rule}: cosine vs plain oracle {oa.cosine(got, want):.7f}, vs P-requantising oracle {oa.cosine(got, mirror):.7f}", flush=True)
 
 
 def test_mxfp8_gemm_swiglu_ffn_shape(cuda):

@@ -34,6 +34,19 @@ def test_rearrange_bit_exact_and_round_trip(cuda, grid, layout):
     assert torch.equal(got.cpu(), orf.rearrange_with_remaining(x, (t, h, w), None, layout))
     back = rf.inv_rearrange_with_remaining(got, (t, h, w), (t, h, w), layout)
     assert torch.equal(back.cpu(), x)
+    # the rf_v3 spelling of the inverse (rf_v3.py:22-97)
+    from mindiesd.layers.flash_attn.sparse_flash_attn_rf_v3 import _bsa_inv_rearrange
+    assert torch.equal(_bsa_inv_rearrange(got, t, h, w, layout).cpu(), x)
+
+
+def test_do_tensor_pooling_as_the_reference_writes_it(cuda):
+    """rf_v2.py:340-348: cut along dim 1, pool both parts along dim 2 (avgpool's default layout), join along dim 1."""
+    from mindiesd.layers.flash_attn.sparse_flash_attn_rf_v2 import do_tensor_pooling
+    x = _rand((2, 5, 300, 128), seed=4)
+    got = do_tensor_pooling(x.to(cuda), 2).cpu()
+    want = torch.cat([orf.avgpool(x[:, :2], 128, "BNSD"), orf.avgpool(x[:, 2:], 128, "BNSD")], dim=1)
+    assert got.shape == (2, 5, 3, 128) and torch.equal(got, want)
+    assert torch.equal(do_tensor_pooling(x.to(cuda), 0).cpu(), orf.avgpool(x, 128, "BNSD"))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -146,8 +146,30 @@ def test_fp8_attention_recipes_agree_with_each_other_and_with_plain_attention():
     assert cosine(a, b) > 0.997 and cosine(b, ref) > 0.995 and cosine(a, ref) > 0.995
 
 
+def test_linear_code_rule_closed_forms():
+    """The linear rule writes the E4M3 code 8 (x + 7) + 118 - 56: integers x give exact powers of two, the value read
+    back from the code is 2^floor(x') (1 + frac(x')) with the fraction rounded to eighths, never more than 6.2 % above
+    and (by the rounding) 3.2 % below 2^x' down to the smallest normal, and the code saturates instead of wrapping."""
+    x = np.arange(-13, 2, dtype=np.float32)                       # x' = x + 7.75 in [-5.25, 8.75]
+    y = np.float32(8.0) * x + oq.L_SEED
+    vals = oq.e4m3_decode(oq.linear_p_codes(y)).astype(np.float64)
+    assert np.array_equal(oq.linear_p_codes(y), (8 * (x + 14.75)).astype(np.uint8))
+    assert np.allclose(vals, np.exp2(np.floor(x + 7.75)) * 1.75)  # frac(x') = 0.75 -> mantissa 6/8
+    rng = np.random.default_rng(0)
+    xr = rng.uniform(-13.5, 1.0, 100000).astype(np.float32)
+    v = oq.e4m3_decode(oq.linear_p_codes(np.float32(8.0) * xr + oq.L_SEED)).astype(np.float64)
+    ratio = v / np.exp2(xr.astype(np.float64) + 7.75)
+    assert ratio.max() <= 1.062 * (1 + 2.0 ** -4) and ratio.min() >= 1 - 2.0 ** -4
+    assert abs(ratio.mean() - 1.04) < 0.005 and ratio.std() < 0.035
+    # largest code the kernel can reach: score = reference + threshold -> 126 (= 448), never the NaN code 127
+    assert oq.linear_p_codes(np.float32(8.0) * oq.L_TAU + oq.L_SEED) == 126
+    assert np.array_equal(oq.linear_p_codes(np.array([-1e9, -np.inf, np.nan, 0.49, 0.5, 1.5, 2.5, 1e9], np.float32)),
+                          np.array([0, 0, 0, 0, 0, 2, 2, 255], np.uint8))
+
+
+@pytest.mark.parametrize("p_rule", ["linear", "exp2"])
 @pytest.mark.parametrize("pow2", [False, True])
-def test_requantised_probabilities_stay_within_a_bound_of_the_plain_form(pow2):
+def test_requantised_probabilities_stay_within_a_bound_of_the_plain_form(pow2, p_rule):
     """``fp8_attention(requant_p=True)`` (P rounded to E4M3 per 128-key tile, denominator from the rounded values,
     lazily moved reference) against the plain quantise -> dequantise form: an E4M3 probability carries at most
     2^-4 relative error, and the errors of a row average out over its keys - the outputs differ by far less than
@@ -160,14 +182,14 @@ def test_requantised_probabilities_stay_within_a_bound_of_the_plain_form(pow2):
     q, k, v = make(), make(), make()
     k[:, :, 300:] *= 1.5            # rising row maxima: the reference has to move after the first tile
     a = oq.fp8_attention(q, k, v, pow2=pow2).float()
-    b = oq.fp8_attention(q, k, v, pow2=pow2, requant_p=True).float()
+    b = oq.fp8_attention(q, k, v, pow2=pow2, requant_p=True, p_rule=p_rule).float()
     assert torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0) >= 0.9999
     assert (a - b).abs().max() <= 2.0 ** -5 * v.float().abs().max()
     # one key tile, uniform scores: every probability is the same power of two, the rounding is exact and the
     # result is the mean of the (de)quantised values whatever the recipe does with the reference
     kz = torch.zeros(1, 1, 100, 128, dtype=torch.bfloat16)
     vz = make()[:, :1, :100]
-    out = oq.fp8_attention(q[:, :1, :40], kz, vz, pow2=pow2, requant_p=True).float()
+    out = oq.fp8_attention(q[:, :1, :40], kz, vz, pow2=pow2, requant_p=True, p_rule=p_rule).float()
     codes, sc = oq.per_channel_quant(vz)
     mean = (torch.from_numpy(oq.e4m3_decode(codes.numpy())) * sc[..., None, :]).mean(dim=-2, keepdim=True)
     assert (out - mean.to(torch.bfloat16).float()).abs().max() <= 2.0 ** -7 * mean.abs().max()
