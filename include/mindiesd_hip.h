@@ -129,8 +129,9 @@ int mindiesd_block_sparse_attention_general_fwd(const void* q, const void* k, co
  * on the device; pass 1 computes, per pair, the key blocks both partners selected with one 256-row workgroup (each
  * K/V tile is fetched once for both, the dense kernel's inner loop); pass 2 adds, per query block, the key blocks
  * only it selected, continuing the running softmax of pass 1.  Same semantics as
- * mindiesd_block_sparse_attention_fwd on the lists of the mask (results differ by the order of the accumulation
- * only); replaces the same reference kernels.  token_order (optional, self-attention): as in the gather entry
+ * mindiesd_block_sparse_attention_fwd on the lists of the mask; results differ by the order of the accumulation and
+ * by one more rounding to the 16-bit output type (pass 1 hands its normalised rows to pass 2 through `out`), well
+ * inside the reference kernels' 2^-6 rule; replaces the same reference kernels.  token_order (optional, self-attention): as in the gather entry
  * point above.  workspace: mindiesd_block_sparse_attention_paired_workspace_size bytes, 16-byte aligned.
  * Returns 2 when the mask is too large for the pairing kernels (more than 2048 key blocks, or mask rows of one
  * head beyond about 150 KiB of bits); the caller then uses the list entry points. */

@@ -10,7 +10,8 @@
 //
 // No counterpart in the reference (its sparse kernels are closed vendor binaries behind
 // csrc/plugin/block_sparse_attention.cpp:31-121); the result of the attention does not depend on the pairing
-// except for the order of the floating-point accumulation.
+// except for the order of the floating-point accumulation and for one rounding: the first pass leaves its
+// normalised rows in the 16-bit output tensor, from where the second pass takes them up again.
 //
 // bsa_bits_kernel:       int8 mask rows -> bit rows + their popcounts.
 // bsa_candidates_kernel: per query block the kCand blocks of the same head with the largest similarity

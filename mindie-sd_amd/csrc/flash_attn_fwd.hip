@@ -93,7 +93,9 @@ __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu
 // INIT (block-sparse only): second pass of the paired scheme - the output rows and p.state already hold the
 // normalised result and the log-sum-exp of the key blocks covered by the first pass; the running softmax starts
 // from them (maximum = that log-sum-exp, sum = 1) instead of from nothing, and a query block without further key
-// blocks is left as it is.
+// blocks is left as it is.  The first pass stores its rows in the 16-bit output type, so a row with key blocks in
+// both passes is rounded to 16 bits once more than a one-pass walk would round it (a relative 2^-9 for bf16 on
+// the first pass's share of the row).
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false,
           bool INIT = false>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
@@ -204,9 +206,13 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
       const int qrow = q0 + wave * QPW + l32;
       const bool ok = qrow < Sq;
       const int orow = GATHER ? p.tok[ok ? qrow : 0] : (ok ? qrow : 0);
-      const float lse2 = ok ? p.state[(long long)bn * p.Sq + qrow] : 0.f;
+      // A first pass that saw only non-finite scores leaves -inf: such a row starts from nothing at reference 0
+      // (a seed of +inf would turn every score into NaN).
+      const float lse_in = ok ? p.state[(long long)bn * p.Sq + qrow] : 0.f;
+      const bool have = lse_in > -INFINITY;
+      const float lse2 = have ? lse_in : 0.f;
       m_run[0] = lse2;
-      l_run[0] = h == 0 ? 1.f : 0.f;  // the two halves of a row add up their sums at the end
+      l_run[0] = (h == 0 && have) ? 1.f : 0.f;  // the two halves of a row add up their sums at the end
 #pragma unroll
       for (int r = 0; r < 16; ++r) negm[0][r] = -lse2;
       const T* orow_p = og + (long long)orow * p.o_ss;
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         for (int g = 0; g < 4; ++g) {
           const typename E::x4 pk = *(const typename E::x4*)(orow_p + db * 32 + 8 * g + 4 * h);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) oacc[db][0][4 * g + j] = ok ? (float)pk[j] : 0.f;
+          for (int j = 0; j < 4; ++j) oacc[db][0][4 * g + j] = (ok && have) ? (float)pk[j] : 0.f;
         }
     }
   }
@@ -1048,7 +1054,8 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
 // Block-sparse attention driven by the int8 mask itself, in two passes over paired query blocks (bsa_pair.hip):
 // pairing + lists, then the key blocks both partners of a pair selected (256-row workgroups, the dense kernel's
 // inner loop), then what only one of them selected, continuing the running softmax.  Same result as
-// mindiesd_block_sparse_attention_fwd on the lists of the mask up to the order of accumulation.
+// mindiesd_block_sparse_attention_fwd on the lists of the mask up to the order of accumulation and one more
+// rounding to the 16-bit output type: the first pass hands its normalised rows to the second through `out`.
 size_t mindiesd_block_sparse_attention_paired_workspace_size(int B, int N, int Sq, int Skv) {
   if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return 0;
   const long long BN = (long long)B * N;

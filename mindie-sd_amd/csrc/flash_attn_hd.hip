@@ -12,7 +12,10 @@
 // O^T += V^T P^T on the 32x32x16 matrix instruction, P^T straight from the score accumulators, V^T by the
 // transposing LDS read), with a plain data path instead of the tuned one: K/V tiles of BN keys go through registers
 // into LDS (requested one tile ahead, zero-filled beyond head_dim and beyond the sequence, rows padded by 16 bytes
-// against bank conflicts), two LDS stages, one barrier per tile; the running maximum moves with every tile.
+// against bank conflicts), two LDS stages, one barrier per tile.  The reference maximum of the running softmax is
+// moved lazily, as in flash_attn_fwd.hip: only when some row of the wave exceeds it by more than 2^kTauHd (or sees
+// its first visible key); the score accumulators are seeded with minus the reference, so the exponential applies
+// to the matrix result directly and a tile without a move costs no rescaling of the output accumulators.
 #include "common.hpp"
 #include "fa_params.hpp"
 
@@ -22,7 +25,7 @@ template <int DP>
 struct HdCfg {
   static constexpr int kNW = 4;                      // waves per workgroup, 32 query rows each
   static constexpr int kBM = kNW * 32;
-  static constexpr int kBN = DP <= 128 ? 64 : 32;    // keys per tile
+  static constexpr int kBN = DP <= 64 ? 128 : (DP <= 128 ? 64 : 32);  // keys per tile
   static constexpr int kNKB = kBN / 32;
   static constexpr int kCols = DP / 8;               // 16-byte chunks per row
   static constexpr int kRowBytes = DP * 2 + 16;
@@ -34,6 +37,8 @@ struct HdCfg {
   static constexpr int kChunksPerThread = kBN * kCols / (kNW * 64);
   static_assert(kBN * kCols % (kNW * 64) == 0, "tile chunks must split evenly over the threads");
 };
+
+constexpr float kTauHd = 8.0f;  // probabilities stay below 2^8: exact in fp32, representable in bf16 and fp16
 
 template <int DT, int DP>
 __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const FaParams p, const int D) {
@@ -105,7 +110,12 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   for (int db = 0; db < kDB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  // m_run: reference maximum (log2 units) the sums and outputs are expressed in, -inf until the row has seen a
+  // visible key; negm: minus that reference (0 while it is -inf) in the 16 slots that seed a score accumulator
   float m_run = -INFINITY, l_run = 0.f;
+  f32x16_t negm;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) negm[r] = 0.f;
 
   // ---- tile staging: thread t owns chunks t, t + 256, ... of the K tile and of the V tile ---------------------------
   i32x4_t kreg[C::kChunksPerThread], vreg[C::kChunksPerThread];
@@ -156,15 +166,11 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
     // ---- S^T = K Q^T --------------------------------------------------------------------------------------------
     f32x16_t sacc[C::kNKB];
 #pragma unroll
-    for (int kb = 0; kb < C::kNKB; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-#pragma unroll
     for (int ks = 0; ks < kKS; ++ks)
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb) {
         const X8 a = *(MSD_LDS const X8*)(kb_base + (kb * 32 + l32) * C::kRowBytes + (2 * ks + h) * 16);
-        sacc[kb] = E::mfma32(a, qf[ks], sacc[kb]);
+        sacc[kb] = E::mfma32(a, qf[ks], ks == 0 ? negm : sacc[kb]);   // = score - reference
       }
 
     // ---- visibility: end of the sequence, causal diagonal, boolean mask -----------------------------------------
@@ -191,16 +197,30 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
     for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
-    mx = half_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that have not seen a visible key yet
-    const float alpha = fast_exp2(m_run - m_use);
-    m_run = m_new;
-    l_run *= alpha;
+    // mx = the lane's largest score minus the reference (minus 0 while the row has no reference yet).  A lane asks
+    // for a move when its part exceeds the threshold or shows the row its first visible key; some lane of a row
+    // does so iff the row's maximum does.
+    const bool unseen = m_run == -INFINITY;
+    if (__builtin_amdgcn_ballot_w64(unseen ? mx > -INFINITY : mx > kTauHd) != 0) {
+      mx = half_max(mx);
+      // first visible key: the exact row maximum becomes the reference (whatever its sign); later: only upwards
+      float delta = unseen ? mx : fmaxf(mx, 0.f);
+      delta = (delta == -INFINITY) ? 0.f : delta;
+      // (a row without a reference has zero sums and outputs: factor 1, not 2^-delta, which may overflow)
+      const float alpha = unseen ? 1.f : fast_exp2(-delta);
+      if (!unseen || mx > -INFINITY) m_run = (unseen ? 0.f : m_run) + delta;
+      l_run *= alpha;
 #pragma unroll
-    for (int db = 0; db < kDB; ++db)
+      for (int r = 0; r < 16; ++r) negm[r] = m_run == -INFINITY ? 0.f : -m_run;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+      for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[kb][r] -= delta;
+#pragma unroll
+      for (int db = 0; db < kDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
     X8 pf[C::kNKB][2];
     float ls = 0.f;
 #pragma unroll
@@ -209,7 +229,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
       for (int t2 = 0; t2 < 2; ++t2) {
         X8 pk;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) pk[j] = E::from_float(fast_exp2(sacc[kb][8 * t2 + j] - m_use));
+        for (int j = 0; j < 8; ++j) pk[j] = E::from_float(fast_exp2(sacc[kb][8 * t2 + j]));
         pf[kb][t2] = pk;
         ls = E::sum8(pk, ls);  // the sum of the rounded probabilities, the values the second product uses
       }

@@ -96,12 +96,14 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
     return (out, lse) if return_lse else out
 
 
-def _varlen_meta(cu_q, cu_k, total_q, total_k, device):
+def _varlen_meta(cu_q, cu_k, total_q, total_k, device, max_q=None, max_k=None):
     """Cumulative lengths -> (int32 [B, 4] device table {first query token, query count, first key token, key
     count}, longest query count, longest key count, B).  Host lists / CPU tensors are validated and give exact
     bounds; device tensors are turned into the table on the device without a host synchronisation - the bounds
-    are then the token totals (workgroups past a sequence's end return at once) and the entries are clamped to the
-    tensors instead of validated."""
+    are then the token totals (workgroups past a sequence's end return at once) unless the caller names the longest
+    sequences (``max_q`` / ``max_k``), and the entries are clamped to the tensors instead of validated: a malformed
+    device table cannot be rejected without reading it back, so it yields clamped sequences, never an access outside
+    the tensors."""
     on_device = isinstance(cu_q, torch.Tensor) and cu_q.is_cuda and isinstance(cu_k, torch.Tensor) and cu_k.is_cuda
     if on_device:
         if cu_q.dim() != 1 or cu_k.dim() != 1 or cu_q.shape[0] != cu_k.shape[0] or cu_q.shape[0] < 2:
@@ -112,7 +114,12 @@ def _varlen_meta(cu_q, cu_k, total_q, total_k, device):
         lk = (ck[1:] - ck[:-1]).clamp(min=0)
         lq, lk = torch.minimum(lq, total_q - sq0), torch.minimum(lk, total_k - sk0)
         meta = torch.stack([sq0, lq, sk0, lk], dim=1).to(torch.int32).contiguous()
-        return meta, total_q, max(total_k, 1), cq.shape[0] - 1
+        bound_q = total_q if max_q is None else max(min(int(max_q), total_q), 1)
+        bound_k = total_k if max_k is None else min(int(max_k), total_k)
+        if max_q is not None or max_k is not None:   # the named bounds hold whatever the table says
+            meta = torch.stack([sq0, lq.clamp(max=bound_q), sk0, lk.clamp(max=max(bound_k, 0))], dim=1) \
+                .to(torch.int32).contiguous()
+        return meta, bound_q, max(bound_k, 1), cq.shape[0] - 1
     def lengths(cu, name):
         vals = [int(x) for x in (cu.detach().cpu().tolist() if isinstance(cu, torch.Tensor) else cu)]
         if len(vals) < 2 or vals[0] != 0 or any(b < a for a, b in zip(vals, vals[1:])):
@@ -133,18 +140,24 @@ def _varlen_meta(cu_q, cu_k, total_q, total_k, device):
     return meta_t, max(seqlens_q), max(max(seqlens_k), 1), len(seqlens_q)
 
 
-def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=False):
+def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=False, max_seqlen_q=None,
+                           max_seqlen_k=None):
     """Packed sequences: q [Tq, N, D], k / v [Tk, Nkv, D]; ``cu_seqlens_q`` / ``cu_seqlens_k``: cumulative sequence
     lengths (batch + 1 entries; lists, CPU tensors or device tensors - the latter are used without a host
-    synchronisation).  Returns [Tq, N, D]."""
+    synchronisation).  Returns [Tq, N, D].  Host tables are validated (ParametersInvalid).  Device tables are
+    clamped to the tensors instead; query rows that no sequence of such a table covers come back as zeros, and
+    ``max_seqlen_q`` / ``max_seqlen_k`` (optional, device tables only) bound the launch to the longest sequence
+    instead of the token totals."""
     _check_qkv(q, k, v)
     if q.dim() != 3 or k.shape != v.shape or k.dim() != 3 or q.shape[1] % k.shape[1] != 0:
         raise ParametersInvalid("Inconsistent query/key/value shapes.")
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
-    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    unchecked = isinstance(cu_seqlens_q, torch.Tensor) and cu_seqlens_q.is_cuda
+    out = (torch.zeros if unchecked else torch.empty)(q.shape, dtype=q.dtype, device=q.device)
     if q.shape[0] == 0:
         return out
-    meta_t, max_q, max_k, nseq = _varlen_meta(cu_seqlens_q, cu_seqlens_k, q.shape[0], k.shape[0], q.device)
+    meta_t, max_q, max_k, nseq = _varlen_meta(cu_seqlens_q, cu_seqlens_k, q.shape[0], k.shape[0], q.device,
+                                              max_seqlen_q, max_seqlen_k)
     if max_q == 0:
         return out
     tn = lambda t: (0, t.stride(1), t.stride(0))  # (batch, head, token) strides of a [T, N, D] tensor

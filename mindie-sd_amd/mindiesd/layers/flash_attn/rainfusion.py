@@ -9,6 +9,8 @@ the inverse permutation.  Every function keeps the reference's signature and lay
 """
 import math
 
+import threading
+
 import torch
 
 from .hip_flash_attn import HEAD_DIM, _strides_bns
@@ -267,31 +269,54 @@ def get_blockwise_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_sha
 # ------------------------------------------------------------------------------------------------
 # block-sparse attention kernels (rf_v2.py:351-381, rf_v3.py:122-190)
 # ------------------------------------------------------------------------------------------------
-_token_order_cache = {}
+_token_order_cache = {}            # key -> (table, event or None once the fill is known to have finished)
+_token_order_lock = threading.Lock()
+
+
+def _build_token_order(t, h, w, txt_len, dev):
+    s = t * h * w + txt_len
+    tok = torch.empty((s,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _native.lib().mindiesd_rf_token_order(tok.data_ptr(), s, t, h, w, txt_len, _native.stream_ptr(dev))
+    _native.check(rc, "mindiesd_rf_token_order")
+    return tok
 
 
 def token_order(latent_shape, txt_len, device):
     """int32 [t*h*w + txt_len]: row of the original [text | image] sequence that holds the token at position i
     of RainFusion's [image in 8x8-window order | text] sequence (the index map of rearrange_with_remaining,
-    rf_v2.py:137-196, 297-312).  Built once per (grid, text length, device)."""
+    rf_v2.py:137-196, 297-312).  Built once per (grid, text length, device) by a small kernel on the current
+    stream and kept; the host never waits for it.  A later call on another stream is ordered after the fill by an
+    event.  Under HIP graph capture a table whose fill is not yet known to be over is not reused: the call builds
+    its own inside the graph (a kernel node like any other), so a first call for a grid can be captured."""
     t, h, w = (int(v) for v in latent_shape)
+    txt_len = int(txt_len)
     if t <= 0 or h < 8 or w < 8:
         raise ParametersInvalid(f"latent_shape_q must be (t, h, w) with h >= 8 and w >= 8, but got {latent_shape}.")
     dev = torch.device(device)
-    key = (t, h, w, int(txt_len), dev.type, dev.index if dev.index is not None else torch.cuda.current_device())
-    tok = _token_order_cache.get(key)
-    if tok is None:
-        s = t * h * w + int(txt_len)
-        tok = torch.empty((s,), dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _native.lib().mindiesd_rf_token_order(tok.data_ptr(), s, t, h, w, int(txt_len), _native.stream_ptr(dev))
-        _native.check(rc, "mindiesd_rf_token_order")
-        # the table is reused by later calls on whatever stream is current then: wait once, here, for the kernel
-        # that fills it
-        torch.cuda.current_stream(dev).synchronize()
-        if len(_token_order_cache) >= 16:
-            _token_order_cache.clear()
-        _token_order_cache[key] = tok
+    key = (t, h, w, txt_len, dev.type, dev.index if dev.index is not None else torch.cuda.current_device())
+    capturing = torch.cuda.is_current_stream_capturing()
+    with _token_order_lock:
+        entry = _token_order_cache.get(key)
+    if entry is not None:
+        tok, done = entry
+        if done is None:
+            return tok
+        if not capturing:
+            if done.query():
+                with _token_order_lock:
+                    _token_order_cache[key] = (tok, None)
+            else:
+                torch.cuda.current_stream(dev).wait_event(done)
+            return tok
+    tok = _build_token_order(t, h, w, txt_len, dev)
+    if not capturing:
+        done = torch.cuda.Event()
+        done.record(torch.cuda.current_stream(dev))
+        with _token_order_lock:
+            if len(_token_order_cache) >= 16:
+                _token_order_cache.clear()
+            _token_order_cache[key] = (tok, done)
     return tok
 
 

@@ -65,6 +65,46 @@ def test_block_sparse_attention_in_a_graph(cuda):
                         mk(0), [mk(10), mk(20), mk(30)])
 
 
+def test_first_rainfusion_call_of_a_grid_in_a_graph(cuda):
+    """The whole rf_v3 call (permute + pool, mask, pairing, attention through the token table) captured for a latent
+    grid that no earlier call has seen: the token table is then built inside the graph, without a host wait."""
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    warm_grid, grid = (2, 16, 24), (3, 19, 17)      # the second one is used nowhere else in the tests
+    n = 2
+    mk = lambda g, sd: tuple(_rnd((1, n, g[0] * g[1] * g[2], 128), sd + i).to(cuda) for i in range(3))
+    run = lambda g: (lambda q, k, v: rf.bsa_sparse_attention_v3(q, k, v, latent_shape_q=g, sparsity=0.5,
+                                                                input_layout="BNSD")[0])
+    run(warm_grid)(*mk(warm_grid, 0))               # library load and kernel attributes, on another grid
+    torch.cuda.synchronize(cuda)
+    assert not any(key[:3] == grid for key in rf._token_order_cache)
+    static = [t.clone() for t in mk(grid, 1)]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = run(grid)(*static)
+    for step, new in enumerate([mk(grid, 10), mk(grid, 20), mk(grid, 30)]):
+        for dst, src in zip(static, new):
+            dst.copy_(src)
+        graph.replay()
+        got = out.clone()
+        want = run(grid)(*[t.clone() for t in new])  # eager: builds and caches its own table
+        torch.cuda.synchronize(cuda)
+        assert torch.equal(got, want), f"replay {step} differs from the eager call"
+
+
+def test_token_order_is_shared_between_streams_without_a_host_wait(cuda):
+    from mindiesd.layers.flash_attn import rainfusion as rf
+    grid = (2, 11, 13)
+    a = rf.token_order(grid, 5, cuda)
+    side = torch.cuda.Stream(device=cuda)
+    with torch.cuda.stream(side):
+        b = rf.token_order(grid, 5, cuda)           # same table, ordered after its fill by an event
+        on_side = b.clone()
+    side.synchronize()
+    torch.cuda.synchronize(cuda)
+    assert a.data_ptr() == b.data_ptr() and torch.equal(on_side, a)
+    assert sorted(a.cpu().tolist()) == list(range(2 * 11 * 13 + 5))
+
+
 def test_two_streams_and_two_threads(cuda):
     """Launches from two host threads on two streams at once (no shared state in the library): each result equals the
     one computed alone."""

@@ -109,6 +109,24 @@ def test_attention_forward_varlen(cuda, causal):
     _check(out2, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), scale=0.05, causal=causal))
 
 
+def test_varlen_device_table_uncovered_rows_and_named_bounds(cuda):
+    """Device cu_seqlens cannot be validated without a host read-back: rows that no sequence covers come back as
+    zeros (not as whatever the allocation held), and the optional longest-sequence bounds give the same result."""
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention_varlen
+    lens = [200, 150]                                 # 350 of 400 query tokens are covered
+    cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+    q, k, v = _rand((400, 2, 128), 21), _rand((350, 2, 128), 22), _rand((350, 2, 128), 23)
+    torch.full((400, 2, 128), float("nan"), dtype=torch.bfloat16, device=cuda)   # dirty the allocator's pool
+    torch.cuda.empty_cache()
+    out = flash_attention_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu.to(cuda), cu.to(cuda), 128 ** -0.5).cpu()
+    ref = attention_varlen(q[:350], k, v, cu.tolist(), cu.tolist())
+    _check(out[:350], ref)
+    assert (out[350:] == 0).all()
+    out2 = flash_attention_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu.to(cuda), cu.to(cuda), 128 ** -0.5,
+                                  max_seqlen_q=200, max_seqlen_k=200).cpu()
+    assert torch.equal(out2, out)
+
+
 def test_varlen_single_sequence_equals_dense(cuda):
     import mindiesd
     q, k, v = _rand((700, 2, 128), 14, mul=0.5), _rand((700, 2, 128), 15, mul=0.5), _rand((700, 2, 128), 16, mul=0.5)

@@ -59,6 +59,41 @@ def test_static_scratch_matches_workspace_entry_point(cuda):
     assert torch.equal(got_s, want_s) and torch.equal(got8, want8)
 
 
+def test_static_entry_point_under_graph_capture_allocates_nothing(cuda):
+    """The callers the entry point is for: a call recorded into a HIP graph (after one eager call, which resolves the
+    array's address), replayed on new values with eager calls of the workspace entry point in between; the
+    allocator's byte count does not move across a call."""
+    from mindiesd import _native
+    lib = _native.lib()
+    b, n, s, d = 1, 3, 700, 128
+    s128 = (s + 127) // 128 * 128
+    v = _v((b, n, s, d), 5, torch.bfloat16).to(cuda)
+    v8t = torch.zeros((b, n, d, s128), dtype=torch.uint8, device=cuda)
+    scale = torch.zeros((b, n, d), dtype=torch.float32, device=cuda)
+
+    def call():
+        return lib.mindiesd_fp8_v_quant_static(v.data_ptr(), v8t.data_ptr(), scale.data_ptr(),
+                                               _native.DTYPE_CODE[v.dtype], b, n, s, d, v.stride(0), v.stride(1),
+                                               v.stride(2), _native.stream_ptr(cuda))
+
+    assert call() == 0                                # first call on the device: symbol lookup
+    torch.cuda.synchronize(cuda)
+    before = torch.cuda.memory_allocated(cuda), torch.cuda.memory_reserved(cuda)
+    assert call() == 0
+    torch.cuda.synchronize(cuda)
+    assert (torch.cuda.memory_allocated(cuda), torch.cuda.memory_reserved(cuda)) == before
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        assert call() == 0
+    for seed in (6, 7, 8):
+        new = (_v((b, n, s, d), seed, torch.bfloat16) * (seed - 5.5)).to(cuda)
+        v.copy_(new)
+        graph.replay()
+        got8, got_s = v8t.clone(), scale.clone()
+        (want8, want_s), _ = _both(lib, new, _native)  # eager work between the replays
+        assert torch.equal(got_s, want_s) and torch.equal(got8, want8), f"replay with seed {seed}"
+
+
 def test_static_scratch_limits_and_errors(cuda):
     from mindiesd import _native
     lib = _native.lib()
