@@ -27,9 +27,21 @@ for _p in (ROOT, os.path.join(ROOT, "mindie-sd_amd")):
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes of one dense 14B-720p launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by a 1 GiB copy kernel (summary and commands: profiles/fa_fwd_dense_bf16_wan14b_720p.md)
-DENSE_TRAFFIC_BYTES = 1.71e10
+DENSE_PROFILE = os.path.join(ROOT, "profiles", "fa_fwd_dense_bf16_wan14b_720p.md")
+
+
+def dense_traffic_bytes():
+    """HBM-side bytes of one dense 14B-720p launch (fetch + write) as the committed rocprofv3 summary states them
+    (--pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel); None when the summary is not there."""
+    import re
+    try:
+        with open(DENSE_PROFILE) as f:
+            text = f.read()
+        head = text[text.index("### the headline launch"):]
+        m = re.search(r"fetch ([0-9.]+) GB.*?write ([0-9.]+) GB", head)
+        return (float(m.group(1)) + float(m.group(2))) * 1e9
+    except (OSError, ValueError, AttributeError):
+        return None
 
 # workloads
 CFG_14B_720P = dict(B=1, N=40, S=75600, D=128, grid=(21, 45, 80))
@@ -247,7 +259,10 @@ def extra_sparse(device, steps, warmup, dense_ms):
         "attention_kernel_ms": km, "attention_kernel_tflops_actual": f * density / km / 1e9,
         "attention_kernel_speedup_vs_dense": dense_ms / km,
         "one_pass_list_kernel_ms": median(list_ms),
+        # HBM-bound pass: algorithmic bytes = q, k, v read once and written once in window order (+ the pooled blocks)
         "permute_pool_ms": median(perm_ms), "permute_pool_gbs": 6 * 774.144e6 / median(perm_ms) / 1e6,
+        "permute_pool_algorithmic_gb": 6 * 0.774144,
+        "permute_pool_frac_of_hbm_peak": 6 * 774.144e6 / median(perm_ms) / 1e6 / PEAK_HBM_GBS,
         "mask_ms": median(mask_ms),
         "topk_only_mask_density": density25,
         "topk_only_pipeline_ms": median(full25_ms), "topk_only_speedup_vs_dense": dense_ms / median(full25_ms),
@@ -336,12 +351,17 @@ def extra_fp8(device, steps, warmup):
     bm, km, qm, em = median(bf16_ms), median(kern_ms), median(quant_ms), median(e2e_ms)
     # quantisation pass: read q, k once and v twice (maximum, then quantise), write one byte per element
     quant_bytes = (4 * 2 + 3 * 1) * cfg["N"] * cfg["S"] * cfg["D"]
+    alg_bytes = (3 * 2 + 3 * 1) * cfg["N"] * cfg["S"] * cfg["D"]
     return {"workload": "FP8 attention B1 N40 S32760 D128, N(0,1) with 1% x8 outliers; Q,K per-128-token scales "
                         "(amax/448), V per-channel, P e4m3 per tile (linear code rule)",
             "bf16_ms": bm, "bf16_tflops": f / bm / 1e9,
             "fp8_kernel_ms": km, "fp8_kernel_tflops": f / km / 1e9, "fp8_kernel_frac_of_fp8_peak": f / km / 1e9 / PEAK_FP8_TFLOPS,
             "fp8_kernel_speedup_vs_bf16": bm / km,
+            # HBM-bound pass.  quant_pass_gbs counts what the kernels move (V is read twice: maximum, then codes);
+            # the roofline fraction prices the algorithmic bytes: q, k, v read once, one byte per element written
             "quant_pass_ms": qm, "quant_pass_gbs": quant_bytes / qm / 1e6,
+            "quant_pass_algorithmic_gb": alg_bytes / 1e9,
+            "quant_pass_frac_of_hbm_peak": alg_bytes / qm / 1e6 / PEAK_HBM_GBS,
             "fp8_end_to_end_ms": em, "fp8_end_to_end_speedup_vs_bf16": bm / em,
             "cosine_fp8_vs_unquantised_bf16_kernel": cos,
             "exp2_rule_kernel_ms": median(xkern_ms), "exp2_rule_kernel_speedup_vs_bf16": bm / median(xkern_ms),
@@ -351,6 +371,8 @@ def extra_fp8(device, steps, warmup):
             "pow2_recipe_cosine_vs_unquantised_bf16_kernel": cos_p,
             "rotated_end_to_end_ms": median(rot_ms), "rotated_end_to_end_speedup_vs_bf16": bm / median(rot_ms),
             "rotate_quant_qk_fused_ms": median(rq_ms), "rotate_quant_qk_matmul_then_quant_ms": median(mm_ms),
+            # q and k read once (2 B), one code byte written per element
+            "rotate_quant_qk_frac_of_hbm_peak": 2 * 3 * cfg["N"] * cfg["S"] * cfg["D"] / median(rq_ms) / 1e6 / PEAK_HBM_GBS,
             "cosine_rotated_fp8_vs_unquantised_bf16_kernel": cos_rot,
             "rotated_pow2_end_to_end_ms": median(rotp_ms), "rotated_pow2_end_to_end_speedup_vs_bf16": bm / median(rotp_ms),
             "cosine_rotated_pow2_fp8_vs_unquantised_bf16_kernel": cos_rotp}
@@ -374,6 +396,8 @@ def extra_gemm(device, steps, warmup):
     return {"workload": "MXFP8 GEMM + SwiGLU M32760 K5120 N2x13824, x N(0,1), w N(0,0.02)",
             "gemm_ms": gm, "gemm_tflops": flops / gm / 1e9, "gemm_frac_of_fp8_peak": flops / gm / 1e9 / PEAK_FP8_TFLOPS,
             "act_quant_ms": qm, "act_quant_gbs": (m * k * 3 + m * k / 32) / qm / 1e6,
+            "act_quant_algorithmic_gb": (m * k * 3 + m * k / 32) / 1e9,
+            "act_quant_frac_of_hbm_peak": (m * k * 3 + m * k / 32) / qm / 1e6 / PEAK_HBM_GBS,
             "with_act_quant_ms": gm + qm}
 
 
@@ -433,9 +457,9 @@ def main():
                                "BNSD, q/k/v = 0.5*N(0,1) seeded"},
         "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": DENSE_TRAFFIC_BYTES,
-                     "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this launch, scaled by a "
-                                       "1 GiB copy (profiles/fa_fwd_dense_bf16_wan14b_720p.md); not re-measured per run",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": dense_traffic_bytes(),
+                     "traffic_source": "read from profiles/fa_fwd_dense_bf16_wan14b_720p.md: rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this launch, scaled by a 1 GiB copy; not re-measured per run",
                      "kernel": "fa_fwd16_kernel<bf16, 8 waves x 32 rows, 128-key tiles>",
                      "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms},
     }
