@@ -144,53 +144,83 @@ struct MaskParams {
 
 constexpr int kMaxBlocks = 2048;
 
-// One workgroup = one query-block row of one (batch, head).
+// One workgroup = kMaskRows consecutive query-block rows of one (batch, head): the pooled keys of the head are read
+// once for all of them (with one row per workgroup the kernel was bound by those reads: 150 KiB from L2 per row),
+// then the rows are finished one after the other.
+constexpr int kMaskRows = 4;
+
 template <int DT>
 __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using T = typename Elem<DT>::type;
-  __shared__ float qrow[128];
-  __shared__ float xs[kMaxBlocks];            // scaled scores, already rounded to 16 bit
-  __shared__ unsigned short key[kMaxBlocks];  // 16-bit pattern of the rounded probabilities
+  __shared__ float qrow[kMaskRows][128];
   __shared__ double red[256];
+  // per key block (dynamic LDS, 14 + 4 * kMaskRows bytes per block: a row of 591 blocks leaves room for 8
+  // workgroups per CU):
+  extern __shared__ __attribute__((aligned(16))) char mask_lds[];
+  const int NBp = (p.NB + 3) & ~3;
+  double* ex = (double*)mask_lds;                                  // exp(score - maximum)
+  unsigned short* key = (unsigned short*)(mask_lds + (size_t)NBp * 8);   // 16-bit pattern of the rounded probabilities
+  float* xs_all = (float*)(mask_lds + (size_t)NBp * 12);           // [kMaskRows][NBp] scaled scores, rounded to 16 bit
   __shared__ int hist[256];
+  __shared__ int suf[257];
+  __shared__ int wave_cnt[4];
   __shared__ int sel_bin, sel_rem, run_base;
-  const int row = blockIdx.x, bn = blockIdx.y;
+  const int row0 = blockIdx.x * kMaskRows, bn = blockIdx.y;
   const int b = bn / p.N, n = bn - b * p.N;
   const int tid = threadIdx.x;
   const int NB = p.NB;
-  const T* qp = (const T*)p.q_pool + b * p.p_sb + n * p.p_sn + (long long)row * p.p_sblk;
+  const int nrows = min(kMaskRows, NB - row0);
   const T* kp = (const T*)p.k_pool + b * p.p_sb + n * p.p_sn;
-  if (tid < 128) qrow[tid] = (float)qp[tid];
+  for (int i = tid; i < kMaskRows * 128; i += 256) {
+    const int r = i >> 7;
+    const T* qp = (const T*)p.q_pool + b * p.p_sb + n * p.p_sn + (long long)(row0 + min(r, nrows - 1)) * p.p_sblk;
+    qrow[r][i & 127] = (float)qp[i & 127];
+  }
   __syncthreads();
 
   // ---- scores: exact dot -> fp32 -> 16 bit; * scale (fp32) -> 16 bit -----------------------------
   // 16 lanes share one key block: each reads 16 bytes of its pooled row (one coalesced 256-byte row per group)
   // and the 16 partial sums are added with lane exchanges.  Every product and sum is exact in fp64, so the order
   // of summation does not matter.
-  float lmax = -INFINITY;
   const int sub = tid & 15, grp16 = tid >> 4;
-  double qd[8];
+  double qd[kMaskRows][8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) qd[j] = (double)qrow[sub * 8 + j];
+  for (int r = 0; r < kMaskRows; ++r)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qd[r][j] = (double)qrow[r][sub * 8 + j];
   for (int c0 = 0; c0 < NB; c0 += 16) {
     const int c = c0 + grp16;
-    double acc = 0.0;
+    double acc[kMaskRows];
+#pragma unroll
+    for (int r = 0; r < kMaskRows; ++r) acc[r] = 0.0;
     if (c < NB) {
       union { i32x4_t v; T e[8]; } u;
       u.v = *(const i32x4_t*)(kp + (long long)c * p.p_sblk + sub * 8);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc = fma(qd[j], (double)(float)u.e[j], acc);
+      for (int j = 0; j < 8; ++j) {
+        const double kv = (double)(float)u.e[j];
+#pragma unroll
+        for (int r = 0; r < kMaskRows; ++r) acc[r] = fma(qd[r][j], kv, acc[r]);
+      }
     }
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-    if (c < NB) {
-      const float s16 = round16<DT>((float)acc);
-      const float x = round16<DT>(__fmul_rn(s16, p.scale));
-      if (sub == 0) xs[c] = x;
-      lmax = fmaxf(lmax, x);
+    for (int r = 0; r < kMaskRows; ++r) {
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) acc[r] += __shfl_xor(acc[r], o, 64);
+      if (c < NB && sub == 0) {
+        const float s16 = round16<DT>((float)acc[r]);
+        xs_all[r * NBp + c] = round16<DT>(__fmul_rn(s16, p.scale));
+      }
     }
   }
+  __syncthreads();
+
+  for (int rr = 0; rr < nrows; ++rr) {
+  const int row = row0 + rr;
+  const float* xs = xs_all + rr * NBp;
+  float lmax = -INFINITY;
+  for (int c = tid; c < NB; c += 256) lmax = fmaxf(lmax, xs[c]);
   red[tid] = (double)lmax;
   __syncthreads();
   for (int s = 128; s > 0; s >>= 1) {
@@ -201,8 +231,13 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   __syncthreads();
 
   // ---- softmax in fp64, rounded to fp32 and then to 16 bit --------------------------------------
+  // (the exponentials are kept in LDS between the sum and the division: fp64 exp is the longest chain here)
   double lsum = 0.0;
-  for (int c = tid; c < NB; c += 256) lsum += exp((double)xs[c] - mx);
+  for (int c = tid; c < NB; c += 256) {
+    const double e = exp((double)xs[c] - mx);
+    ex[c] = e;
+    lsum += e;
+  }
   red[tid] = lsum;
   __syncthreads();
   for (int s = 128; s > 0; s >>= 1) {
@@ -211,7 +246,7 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   }
   const double denom = red[0];
   for (int c = tid; c < NB; c += 256) {
-    const float pr = (float)(exp((double)xs[c] - mx) / denom);
+    const float pr = (float)(ex[c] / denom);
     const T p16 = Elem<DT>::from_float(pr);
     key[c] = __builtin_bit_cast(unsigned short, p16);  // probabilities are >= 0: bit order == value order
   }
@@ -219,33 +254,43 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   __syncthreads();
 
   // ---- keep_len-th largest value: two-level radix select on the 16-bit patterns -------------------
+  // Per level: histogram of one byte, suffix sums over the 256 bins (one bin per thread, a scan inside the
+  // waves and a combine over the four of them), and the bin in which the wanted rank falls: the one with
+  // suffix(bin) >= need > suffix(bin + 1); the rank inside it is need - suffix(bin + 1).
+  const int lane = tid & 63, wv = tid >> 6;
+  auto pick_bin = [&](int need) {
+    int v = hist[tid];
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_down(v, o, 64);
+      if (lane + o < 64) v += t;
+    }
+    if (lane == 0) wave_cnt[wv] = v;
+    __syncthreads();
+    for (int w2 = wv + 1; w2 < 4; ++w2) v += wave_cnt[w2];
+    suf[tid] = v;
+    if (tid == 0) suf[256] = 0;
+    __syncthreads();
+    // bin 0 also takes what no other bin takes (the scan it replaces stopped there)
+    const bool mine = tid == 0 ? suf[1] < need : (suf[tid] >= need && suf[tid + 1] < need);
+    if (mine) {
+      sel_bin = tid;
+      sel_rem = need - suf[tid + 1];
+    }
+    __syncthreads();
+  };
   for (int c = tid; c < NB; c += 256) atomicAdd(&hist[key[c] >> 8], 1);
   __syncthreads();
-  if (tid == 0) {
-    int need = p.keep_len, bin = 255;
-    for (; bin > 0; --bin) {
-      if (hist[bin] >= need) break;
-      need -= hist[bin];
-    }
-    sel_bin = bin;
-    sel_rem = need;
-  }
-  __syncthreads();
+  pick_bin(p.keep_len);
   const int hi_bin = sel_bin;
+  const int rem = sel_rem;
   hist[tid] = 0;
   __syncthreads();
   for (int c = tid; c < NB; c += 256)
     if ((key[c] >> 8) == hi_bin) atomicAdd(&hist[key[c] & 255], 1);
   __syncthreads();
-  if (tid == 0) {
-    int need = sel_rem, bin = 255;
-    for (; bin > 0; --bin) {
-      if (hist[bin] >= need) break;
-      need -= hist[bin];
-    }
-    sel_bin = bin;
-    run_base = 0;
-  }
+  pick_bin(rem);
+  if (tid == 0) run_base = 0;
   __syncthreads();
   const unsigned thr = ((unsigned)hi_bin << 8) | (unsigned)sel_bin;
 
@@ -255,8 +300,6 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   signed char* mrow = p.mask ? p.mask + row_lin * NB : nullptr;
   int* irow = p.blk_idx ? p.blk_idx + row_lin * p.kb_stride : nullptr;
   long long* irow64 = (p.idx64 && b == 0) ? p.idx64 + ((long long)row * p.N + n) * NB : nullptr;
-  const int lane = tid & 63, wv = tid >> 6;
-  __shared__ int wave_cnt[4];
   for (int c0 = 0; c0 < NB; c0 += 256) {
     const int c = c0 + tid;
     bool keep = false;
@@ -287,6 +330,8 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
     if (p.blk_cnt) p.blk_cnt[row_lin] = total;
     if (p.cnt64 && b == 0) p.cnt64[(long long)row * p.N + n] = total;
   }
+  __syncthreads();
+  }  // rows of the workgroup
 #endif
 }
 
@@ -396,11 +441,12 @@ int mindiesd_rf_block_mask(const void* q_pool, const void* k_pool, int dtype, in
   p.B = B; p.N = N; p.NB = NB; p.kb_stride = kb_stride;
   p.keep_len = keep_len; p.txt_blocks = txt_blocks; p.ff_blocks = ff_blocks; p.keep_diag = keep_diag;
   p.scale = scale;
-  dim3 grid(NB, B * N);
+  dim3 grid((NB + kMaskRows - 1) / kMaskRows, B * N);
+  const size_t lds = (size_t)((NB + 3) & ~3) * (12 + 4 * kMaskRows);  // at most 56 KiB (NB <= kMaxBlocks)
   if (dtype == MSD_DTYPE_BF16)
-    hipLaunchKernelGGL(rf_block_mask_kernel<MSD_DTYPE_BF16>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rf_block_mask_kernel<MSD_DTYPE_BF16>, grid, dim3(256), lds, stream, p);
   else
-    hipLaunchKernelGGL(rf_block_mask_kernel<MSD_DTYPE_F16>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rf_block_mask_kernel<MSD_DTYPE_F16>, grid, dim3(256), lds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
