@@ -46,15 +46,12 @@ def test_config1_full(cuda):
     ref = attention_math(q, k, v, None, 128 ** -0.5, head_first=True)
     out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), head_first=True).cpu()
     _check(out, ref)
-    assert data_compare(out, ref, rel=4e-3), "reference's data_compare rule (threshold widened to one bf16 ulp)"
-    # the same rule at the reference's own threshold 1e-3 (tests/utils/utils/precision_compare.py:89): both sides
-    # round to bf16 (spacing 2^-8 relative), so two correct results differ by one ulp in a share of the elements;
-    # the share that passes is reported, and checked against what the oracle's own two roundings would give
+    # the reference's own rule at its own thresholds (tests/utils/utils/precision_compare.py:89: relative to
+    # max(1, |golden|) within 1e-3 for 99.9 % of the elements, never above 0.1); the share that passes is printed
+    assert data_compare(out, ref), "reference's data_compare rule"
     diff = (out.float() - ref.float()).abs() / ref.float().abs().clamp(min=1.0)
-    frac = float((diff <= 1e-3).float().mean())
-    print(f"config 1: data_compare pass fraction at the reference's threshold 1e-3: {frac:.5f} "
-          f"(at 4e-3: {float((diff <= 4e-3).float().mean()):.5f}), largest relative difference {float(diff.max()):.4f}")
-    assert frac >= 0.97
+    print(f"config 1: data_compare pass fraction at the reference's threshold 1e-3: {float((diff <= 1e-3).float().mean()):.5f}, "
+          f"largest relative difference {float(diff.max()):.4f}")
 
 
 def test_fp16(cuda):
