@@ -180,34 +180,32 @@ __global__ __launch_bounds__(256) void rf_block_mask_kernel(const MaskParams p) 
   __syncthreads();
 
   // ---- scores: exact dot -> fp32 -> 16 bit; * scale (fp32) -> 16 bit -----------------------------
-  // 16 lanes share one key block: each reads 16 bytes of its pooled row (one coalesced 256-byte row per group)
-  // and the 16 partial sums are added with lane exchanges.  Every product and sum is exact in fp64, so the order
-  // of summation does not matter.
-  const int sub = tid & 15, grp16 = tid >> 4;
-  double qd[kMaskRows][8];
-#pragma unroll
-  for (int r = 0; r < kMaskRows; ++r)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) qd[r][j] = (double)qrow[r][sub * 8 + j];
-  for (int c0 = 0; c0 < NB; c0 += 16) {
-    const int c = c0 + grp16;
+  // 4 lanes share one key block: lane `sub` reads the 16-byte chunks sub, sub + 4, sub + 8, sub + 12 of its pooled
+  // row (the four lanes of a block read 64 contiguous bytes per request) and the 4 partial sums are added with two
+  // lane exchanges.  Every product and sum is exact in fp64, so the order of summation does not matter.
+  const int sub = tid & 3, grp4 = tid >> 2;
+  for (int c0 = 0; c0 < NB; c0 += 64) {
+    const int c = c0 + grp4;
     double acc[kMaskRows];
 #pragma unroll
     for (int r = 0; r < kMaskRows; ++r) acc[r] = 0.0;
     if (c < NB) {
-      union { i32x4_t v; T e[8]; } u;
-      u.v = *(const i32x4_t*)(kp + (long long)c * p.p_sblk + sub * 8);
+      union { i32x4_t v; T e[8]; } u[4];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const double kv = (double)(float)u.e[j];
+      for (int i = 0; i < 4; ++i) u[i].v = *(const i32x4_t*)(kp + (long long)c * p.p_sblk + (sub + 4 * i) * 8);
 #pragma unroll
-        for (int r = 0; r < kMaskRows; ++r) acc[r] = fma(qd[r][j], kv, acc[r]);
-      }
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const double kv = (double)(float)u[i].e[j];
+#pragma unroll
+          for (int r = 0; r < kMaskRows; ++r) acc[r] = fma((double)qrow[r][(sub + 4 * i) * 8 + j], kv, acc[r]);
+        }
     }
 #pragma unroll
     for (int r = 0; r < kMaskRows; ++r) {
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) acc[r] += __shfl_xor(acc[r], o, 64);
+      for (int o = 2; o > 0; o >>= 1) acc[r] += __shfl_xor(acc[r], o, 64);
       if (c < NB && sub == 0) {
         const float s16 = round16<DT>((float)acc[r]);
         xs_all[r * NBp + c] = round16<DT>(__fmul_rn(s16, p.scale));
