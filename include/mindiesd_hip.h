@@ -272,9 +272,13 @@ int mindiesd_fp8_v_quant_static(const void* v, void* v8t, float* v_scale, int dt
  *   MSD_FP8_P_EXP2       the probabilities of a tile are 2^(score - reference) by the exponential instruction, rounded
  *                        to E4M3 (the older, slower rule).  Default: the E4M3 code of a probability is computed
  *                        directly as round(8 * (score - reference) + const), i.e. the exponential with its mantissa
- *                        interpolated linearly between powers of two; the denominator is summed from the same codes. */
+ *                        interpolated linearly between powers of two; the denominator is summed from the same codes.
+ *   MSD_FP8_K_BLOCK_256  k_scale holds one scale per 256 keys ([B][N][ceil(Skv/256)], mindiesd_fa_block_quant with
+ *                        block_size 256 - the K recipe of FP8RotateQuantFA, mindiesd/quantization/layer.py:297-302)
+ *                        instead of one per 128. */
 #define MSD_FP8_LOG2_DOMAIN 1
 #define MSD_FP8_P_EXP2 2
+#define MSD_FP8_K_BLOCK_256 4
 int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, const float* q_scale,
                                const float* k_scale, const float* v_scale, void* out, int out_dtype, int B, int N,
                                int Sq, int Skv, int D, long long o_sb, long long o_sn, long long o_ss, float scale,

@@ -30,7 +30,7 @@ enum : int {
 
 enum : int { MSD_DTYPE_BF16 = 0, MSD_DTYPE_F16 = 1 };
 // flag bits of mindiesd_fp8_attention_fwd (the same values as in include/mindiesd_hip.h)
-enum : int { MSD_FP8_LOG2_DOMAIN = 1, MSD_FP8_P_EXP2 = 2 };
+enum : int { MSD_FP8_LOG2_DOMAIN = 1, MSD_FP8_P_EXP2 = 2, MSD_FP8_K_BLOCK_256 = 4 };
 
 // ---- element traits: 16-bit storage type -> MFMA operand type + builtins -------------
 template <int DT>

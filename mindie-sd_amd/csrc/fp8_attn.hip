@@ -340,12 +340,13 @@ struct Fp8Params {
   const unsigned char* k8;
   const unsigned char* v8t;
   const float* q_scale;  // [B][N][ceil(Sq/128)]
-  const float* k_scale;  // [B][N][ceil(Skv/128)]
+  const float* k_scale;  // [B][N][ceil(Skv/128)], or [B][N][ceil(Skv/256)] with k_shift = 1
   const float* v_scale;  // [B][N][128]
   void* o;
   long long o_sb, o_sn, o_ss;
   int B, N, Sq, Skv, S128;
   float scale_log2;  // softmax scale * log2(e)
+  int k_shift;       // a K scale covers 128 << k_shift keys
 };
 
 // Two rules for the E4M3 probabilities of a tile (x = score - reference maximum, in log2 units):
@@ -425,7 +426,8 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   constexpr float kTau = PL ? kTauL : kTau8;
   // read through the constant address space: a scalar load, which does not queue behind the tile requests
   typedef const __attribute__((address_space(4))) float* ConstF;
-  const ConstF k_sc = (ConstF)(uintptr_t)(p.k_scale + (long long)bn * kblocks);
+  const int k_shift = p.k_shift;
+  const ConstF k_sc = (ConstF)(uintptr_t)(p.k_scale + (long long)bn * ((kblocks + (1 << k_shift) - 1) >> k_shift));
 
   f32x16_t oacc[4];
 #pragma unroll
@@ -493,7 +495,7 @@ __global__ __launch_bounds__(512, 2) void fp8_fa_fwd_kernel(const Fp8Params p) {
   float k_sc_cur = n_tiles > 0 ? k_sc[0] : 0.f;
   auto tile_step = [&](const int t, auto stage_c) {
     constexpr int stage = decltype(stage_c)::value;
-    const float k_sc_next = k_sc[t + 1 < n_tiles ? t + 1 : t];
+    const float k_sc_next = k_sc[(t + 1 < n_tiles ? t + 1 : t) >> k_shift];
     // issued after the last tile as well (past the end of the buffers: nobody uses it), so that the number of
     // requests in flight is the same on every path
     load_tile(t + 2, (stage + 2) % 3);
@@ -830,7 +832,7 @@ int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, 
   if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return MSD_ERR_BAD_ARG;
   if (D != 128 || !(scale > 0.f)) return MSD_ERR_UNSUPPORTED;
   if (out_dtype != MSD_DTYPE_BF16 && out_dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
-  if (flags & ~(MSD_FP8_LOG2_DOMAIN | MSD_FP8_P_EXP2)) return MSD_ERR_BAD_ARG;
+  if (flags & ~(MSD_FP8_LOG2_DOMAIN | MSD_FP8_P_EXP2 | MSD_FP8_K_BLOCK_256)) return MSD_ERR_BAD_ARG;
   if (((uintptr_t)q8 | (uintptr_t)k8 | (uintptr_t)v8t | (uintptr_t)out) & 15) return MSD_ERR_BAD_ARG;
   if ((o_sb | o_sn | o_ss) & 7) return MSD_ERR_BAD_ARG;
   const int S128 = (Skv + 127) / 128 * 128;
@@ -841,6 +843,7 @@ int mindiesd_fp8_attention_fwd(const void* q8, const void* k8, const void* v8t, 
   p.o = out; p.o_sb = o_sb; p.o_sn = o_sn; p.o_ss = o_ss;
   p.B = B; p.N = N; p.Sq = Sq; p.Skv = Skv; p.S128 = S128;
   p.scale_log2 = scale * 1.4426950408889634f;
+  p.k_shift = (flags & MSD_FP8_K_BLOCK_256) ? 1 : 0;
   const int q_tiles = (Sq + 255) / 256;
   const int total = B * N * q_tiles;
   const int grid = (total + 7) / 8 * 8;

@@ -35,20 +35,24 @@ def quantize_v_per_channel(value, layout="BNSD"):
 
 LOG2E = 1.4426950408889634
 # flag bits of mindiesd_fp8_attention_fwd (include/mindiesd_hip.h)
-FLAG_LOG2_DOMAIN, FLAG_P_EXP2 = 1, 2
+FLAG_LOG2_DOMAIN, FLAG_P_EXP2, FLAG_K_BLOCK_256 = 1, 2, 4
 P_RULES = ("linear", "exp2")
 
 
 def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_dtype=torch.bfloat16, layout="BNSD",
-                            log2_domain=False, p_rule="linear"):
+                            log2_domain=False, p_rule="linear", k_block=128):
     """Attention on already quantised operands (see ``quantize_v_per_channel`` and ``_block_quant``
     with block 128).  Output [B,N,S,128] ('BNSD') or [B,S,N,128] ('BSND') in ``out_dtype``.
     ``log2_domain``: the query was quantised with ``prescale = scale * log2(e)`` and both q and k with
     power-of-two scales; ``scale`` is then not used.
-    ``p_rule``: how a tile's probabilities become E4M3 - see ``fp8_attention_forward``."""
+    ``p_rule``: how a tile's probabilities become E4M3 - see ``fp8_attention_forward``.
+    ``k_block``: 128 or 256 keys per entry of ``k_scale``."""
     if p_rule not in P_RULES:
         raise ParametersInvalid(f"p_rule must be one of {P_RULES}, but got {p_rule}.")
-    flags = (FLAG_LOG2_DOMAIN if log2_domain else 0) | (FLAG_P_EXP2 if p_rule == "exp2" else 0)
+    if k_block not in (128, 256):
+        raise ParametersInvalid(f"k_block must be 128 or 256, but got {k_block}.")
+    flags = ((FLAG_LOG2_DOMAIN if log2_domain else 0) | (FLAG_P_EXP2 if p_rule == "exp2" else 0)
+             | (FLAG_K_BLOCK_256 if k_block == 256 else 0))
     b, n, sq, d = q8.shape
     skv = k8.shape[2]
     shape = (b, n, sq, d) if layout == "BNSD" else (b, sq, n, d)
@@ -63,7 +67,7 @@ def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_d
 
 
 def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=None, k_rot=None, recipe="amax",
-                          p_rule="linear"):
+                          p_rule="linear", k_block=128):
     """Quantise q, k, v (bf16/fp16, 'BNSD' or 'BSND') and run FP8 attention; output like ``query``.
     ``q_rot`` / ``k_rot`` ([128, 128]): query @ q_rot and key @ k_rot are formed inside the quantisation
     pass (the rotated tensors are never written).
@@ -79,7 +83,10 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=No
     two (at most 6 % above 2^x, 3 % rms after the common factor cancels against the denominator, which is summed
     from the same codes) - one multiply-add and one conversion per score; 'exp2' - 2^(score - reference) by the
     exponential instruction, rounded to E4M3 (slower: two quarter-rate instructions per score).  Both stay inside
-    the FP8 workload's tolerance (cosine >= 0.999 against the quantise -> dequantise path)."""
+    the FP8 workload's tolerance (cosine >= 0.999 against the quantise -> dequantise path).
+    ``k_block``: tokens per K scale, 128 (default, the FP8 workload's recipe) or 256 (the K recipe of the reference's
+    FP8RotateQuantFA, mindiesd/quantization/layer.py:297-302; not together with ``k_rot``, whose fused pass quantises
+    per 128 tokens)."""
     for name, t in (("query", query), ("key", key), ("value", value)):
         if not isinstance(t, torch.Tensor) or t.dim() != 4:
             raise ParametersInvalid(f"The input {name} must be a 4-D torch.Tensor.")
@@ -95,11 +102,14 @@ def fp8_attention_forward(query, key, value, scale=None, layout="BNSD", q_rot=No
         scale = query.shape[-1] ** -0.5
     if recipe not in ("pow2", "amax"):
         raise ParametersInvalid(f"recipe must be 'pow2' or 'amax', but got {recipe}.")
+    if k_block not in (128, 256) or (k_block == 256 and k_rot is not None):
+        raise ParametersInvalid(f"k_block must be 128, or 256 without k_rot, but got {k_block}.")
     p2 = recipe == "pow2"
     pre = float(scale) * LOG2E if p2 else 1.0
     q8, qs = (_block_quant(query, 128, layout, pre, p2) if q_rot is None
               else _rot_block_quant(query, q_rot, layout, pre, p2))
-    k8, ks = (_block_quant(key, 128, layout, 1.0, p2) if k_rot is None
+    k8, ks = (_block_quant(key, k_block, layout, 1.0, p2) if k_rot is None
               else _rot_block_quant(key, k_rot, layout, 1.0, p2))
     v8t, vs = quantize_v_per_channel(value, layout)
-    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout, log2_domain=p2, p_rule=p_rule)
+    return fp8_attention_quantized(q8, qs, k8, ks, v8t, vs, scale, query.dtype, layout, log2_domain=p2, p_rule=p_rule,
+                                   k_block=k_block)

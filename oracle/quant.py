@@ -113,7 +113,7 @@ def per_channel_quant(v):
     return torch.from_numpy(e4m3_encode(vf / sc[..., None, :])), torch.from_numpy(sc)
 
 
-def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False, p_rule="linear"):
+def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False, p_rule="linear", k_block=128):
     """FP8 attention of the Wan2.1-14B 480p workload, BNSD: Q and K quantised per (head, 128-token
     block) over all channels, V per (head, channel); bf16-typed output.
     ``requant_p=False``: the quantise -> dequantise path - everything is dequantised and run through plain
@@ -128,7 +128,8 @@ def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False, p_
     code = rne(8 * (score - reference) + 8 * (7.75 + 7)) saturated to [0, 255] - read back as E4M3 that is
     2^floor(x') * (1 + frac(x')) with frac rounded to eighths, x' = score - reference + 7.75: the exponential with
     its mantissa interpolated linearly between powers of two (code 8 e + m stands for 2^(e-7) (1 + m/8)); the reference
-    moves when a row of the group exceeds it by more than 2^1 (so the code stays <= 126 = 448)."""
+    moves when a row of the group exceeds it by more than 2^1 (so the code stays <= 126 = 448).
+    ``k_block``: tokens per K scale (128; 256 = the K recipe of the reference's FP8RotateQuantFA, layer.py:297-302)."""
     d = query.shape[-1]
     if scale is None:
         scale = d ** -0.5
@@ -136,16 +137,16 @@ def fp8_attention(query, key, value, scale=None, pow2=False, requant_p=False, p_
         # log2-domain recipe: the query carries scale * log2(e), block scales are powers of two; the dequantised
         # scores are then in log2 units, i.e. ln(2) stands where the softmax scale stood
         qc, qs = dynamic_block_quant(query, 128, d, scale * 1.4426950408889634, True)
-        kc, ks = dynamic_block_quant(key, 128, d, 1.0, True)
+        kc, ks = dynamic_block_quant(key, k_block, d, 1.0, True)
         scale = math.log(2.0)
     else:
         qc, qs = dynamic_block_quant(query, 128, d)
-        kc, ks = dynamic_block_quant(key, 128, d)
+        kc, ks = dynamic_block_quant(key, k_block, d)
     vc, vs = per_channel_quant(value)
     if requant_p:
         return _fp8_attention_requant(qc, qs, kc, ks, vc, vs, np.float32(scale * 1.4426950408889634), pow2,
-                                      p_rule).to(query.dtype)
-    qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, 128, d)
+                                      p_rule, k_block).to(query.dtype)
+    qd, kd = dequant_block(qc, qs, 128, d), dequant_block(kc, ks, k_block, d)
     vd = torch.from_numpy(e4m3_decode(vc.numpy())) * vs[..., None, :]
     out = torch.empty(query.shape, dtype=torch.float32)
     for r0 in range(0, query.shape[-2], 2048):
@@ -166,7 +167,7 @@ def linear_p_codes(y):
     return np.clip(np.rint(y), 0, 255).astype(np.uint8)
 
 
-def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2, p_rule="linear"):
+def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2, p_rule="linear", k_block=128):
     """The tile loop behind ``fp8_attention(requant_p=True)`` on the quantised operands (codes + scales)."""
     linear = p_rule == "linear"
     tau = L_TAU if linear else P_TAU
@@ -189,7 +190,7 @@ def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2, p_rule="lin
                     t1 = min(t0 + KEY_TILE, skv)
                     raw = q8[bi, ni, r0:r1] @ k8[bi, ni, t0:t1].T                     # exact sums of code products
                     if pow2:  # the scales are powers of two (applied by the matrix instruction's exponents)
-                        s = (raw * (qsc * ksn[bi, ni, t0 // 128])).astype(np.float32)
+                        s = (raw * (qsc * ksn[bi, ni, t0 // k_block])).astype(np.float32)
                         mx = s.max(axis=1) - m_run
                         if first or (mx > tau).any():
                             delta = mx if first else np.maximum(mx, np.float32(0))
@@ -199,7 +200,7 @@ def _fp8_attention_requant(qc, qs, kc, ks, vc, vs, scale_log2, pow2, p_rule="lin
                             l_run *= alpha
                             o_run *= alpha[:, None]
                     else:     # amax/448 scales folded into the softmax scale of the tile
-                        c = np.float32(np.float32(qsc * scale_log2) * ksn[bi, ni, t0 // 128])
+                        c = np.float32(np.float32(qsc * scale_log2) * ksn[bi, ni, t0 // k_block])
                         s = (raw * c).astype(np.float32)
                         mx = s.max(axis=1)
                         if (mx > m_run + tau).any():

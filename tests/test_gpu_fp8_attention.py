@@ -122,6 +122,30 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe, p_rule):
     assert err_m.max() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("recipe", ["pow2", "amax"])
+@pytest.mark.parametrize("s", [1100, 640])
+def test_fp8_attention_k_scale_per_256_tokens(cuda, s, recipe):
+    """K quantised per 256-token block (the K recipe of the reference's FP8RotateQuantFA, layer.py:297-302): scales from
+    fa_block_quant_preprocess(block_size=256), the kernel takes one scale for two key tiles."""
+    from mindiesd import ParametersInvalid
+    from mindiesd.layers.quant import fp8_attention_forward
+    q, k, v = _outlier_inputs((1, 2, s, 128), seed=s + 1)
+    k[:, :, 256:512] *= 4.0                  # neighbouring 256-blocks with scales far apart
+    out = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), recipe=recipe, k_block=256).cpu()
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", k_block=256)
+    mirror = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True, k_block=256)
+    assert cosine(out, want) >= 0.999 and cosine(out, mirror) >= 0.99999
+    # a different quantisation from the per-128 one - except with power-of-two scales, where a coarser block only
+    # shifts exponents and the dequantised values stay the same
+    other = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), recipe=recipe).cpu()
+    assert torch.equal(out, other) == (recipe == "pow2")
+    with pytest.raises(ParametersInvalid):
+        fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), k_block=64)
+    with pytest.raises(ParametersInvalid):
+        fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), k_block=256,
+                              k_rot=torch.eye(128, dtype=torch.bfloat16, device=cuda))
+
+
 @pytest.mark.parametrize("p_rule", ["linear", "exp2"])
 @pytest.mark.parametrize("recipe", ["pow2", "amax"])
 def test_fp8_attention_scores_far_below_zero(cuda, recipe, p_rule):
