@@ -256,11 +256,18 @@ __global__ __launch_bounds__(256) void channel_amax_kernel(const void* v_, unsig
   float m[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) m[j] = 0.f;
-  for (int r = rgrp; r < rows; r += 16) {
-    float f[8];
-    load8<DT>(v + (long long)(row0 + r) * ss + c16 * 8, f);
+  // 8 rows of a thread are requested before the first one is used (rows past the end read row 0 again)
+  for (int r0 = rgrp; r0 < rows; r0 += 128) {
+    union { i32x4_t v; T e[8]; } u[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) m[j] = fmaxf(m[j], fabsf(f[j]));
+    for (int i = 0; i < 8; ++i) {
+      const int r = r0 + 16 * i;
+      u[i].v = *(const i32x4_t*)(v + (long long)(row0 + (r < rows ? r : 0)) * ss + c16 * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m[j] = fmaxf(m[j], fabsf((float)u[i].e[j]));
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) part[rgrp][c16 * 8 + j] = m[j];
@@ -284,51 +291,57 @@ __host__ __device__ __forceinline__ int v8t_pos(int kk) {
 
 // V [B][N][S][128] -> V8T [B][N][128][S128] bytes + per-channel scale [B][N][128] = amax/448.
 // One workgroup = 128 keys of one (batch, head): every channel row it writes is one full 128-byte line.
+// A thread takes 8 channels of two groups of 4 consecutive keys: 4 consecutive keys are 4 consecutive positions of
+// V8T (v8t_pos), so their codes of one channel leave as one dword.  LDS tile [channel][128 positions], 16-byte chunk
+// c of a row stored at chunk c ^ ((channel >> 3) & 7): the 16 threads of a key group, 8 channels apart, then write
+// to 8 different bank groups.
 template <int DT>
 __global__ __launch_bounds__(256) void v_quant_transpose_kernel(const void* v_, const unsigned* amax_bits,
                                                                 unsigned char* v8t, float* vscale, long long sb,
                                                                 long long sn, long long ss, int N, int S, int S128) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using T = typename Elem<DT>::type;
-  __shared__ __attribute__((aligned(16))) unsigned char tile[128][128 + 16];  // [channel][position], padded rows
+  __shared__ __attribute__((aligned(16))) unsigned char tile[128 * 128];
   const int grp = blockIdx.x, bn = blockIdx.y, b = bn / N, n = bn - b * N;
   const T* v = (const T*)v_ + b * sb + n * sn;
-  const int c16 = threadIdx.x & 15, rgrp = threadIdx.x >> 4;
+  const int c16 = threadIdx.x & 15, qd = threadIdx.x >> 4;
   float sc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const float a = __builtin_bit_cast(float, amax_bits[(long long)bn * 128 + c16 * 8 + j]);
     sc[j] = a > 0.f ? __fdiv_rn(a, kE4M3Max) : 1.0f;
   }
-  if (grp == 0 && rgrp == 0) {
+  if (grp == 0 && qd == 0) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) vscale[(long long)bn * 128 + c16 * 8 + j] = sc[j];
   }
-  // all 8 rows of this thread are requested before the first one is used
-  union { i32x4_t v; T e[8]; } u[8];
+  // keys 4 * qd + j and 64 + 4 * qd + j (j < 4): all 8 rows are requested before the first one is used
+  union { i32x4_t v; T e[8]; } u[2][4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int key = grp * 128 + rgrp + 16 * i;
-    u[i].v = i32x4_t{0, 0, 0, 0};
-    if (key < S) u[i].v = *(const i32x4_t*)(v + (long long)key * ss + c16 * 8);
-  }
+  for (int half = 0; half < 2; ++half)
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int kk = rgrp + 16 * i;
-    const int pos = (kk & 64) + v8t_pos(kk & 63);
+    for (int j = 0; j < 4; ++j) {
+      const int key = grp * 128 + half * 64 + 4 * qd + j;
+      u[half][j].v = i32x4_t{0, 0, 0, 0};
+      if (key < S) u[half][j].v = *(const i32x4_t*)(v + (long long)key * ss + c16 * 8);
+    }
+  const int swz = c16 & 7;  // (channel >> 3) & 7 of this thread's channels
 #pragma unroll
-    for (int j = 0; j < 8; j += 4) {
-      const int w = pack4_e4m3(__fdiv_rn((float)u[i].e[j], sc[j]), __fdiv_rn((float)u[i].e[j + 1], sc[j + 1]),
-                               __fdiv_rn((float)u[i].e[j + 2], sc[j + 2]), __fdiv_rn((float)u[i].e[j + 3], sc[j + 3]));
+  for (int half = 0; half < 2; ++half) {
+    const int pos = half * 64 + v8t_pos(4 * qd);  // multiple of 4
+    const int off = (((pos >> 4) ^ swz) << 4) + (pos & 15);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) tile[c16 * 8 + j + e][pos] = (unsigned char)((unsigned)w >> (8 * e));
+    for (int c = 0; c < 8; ++c) {
+      const int w = pack4_e4m3(__fdiv_rn((float)u[half][0].e[c], sc[c]), __fdiv_rn((float)u[half][1].e[c], sc[c]),
+                               __fdiv_rn((float)u[half][2].e[c], sc[c]), __fdiv_rn((float)u[half][3].e[c], sc[c]));
+      *(int*)&tile[(c16 * 8 + c) * 128 + off] = w;
     }
   }
   __syncthreads();
   // 128 channel rows x 128 bytes: 8 lanes write one row
   for (int i = threadIdx.x; i < 128 * 8; i += 256) {
     const int ch = i >> 3, part = i & 7;
-    const i32x4_t w = *(const i32x4_t*)&tile[ch][part * 16];
+    const i32x4_t w = *(const i32x4_t*)&tile[ch * 128 + ((part ^ ((ch >> 3) & 7)) << 4)];
     *(i32x4_t*)(v8t + ((long long)bn * 128 + ch) * S128 + grp * 128 + part * 16) = w;
   }
 #endif
