@@ -145,6 +145,37 @@ def test_block_quant_random(cuda, seed):
     assert bool(((got == wc) | zero).all()), (n, s, dtype, kind, layout, pow2, pre)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_fp8_attention_random_shape(cuda, seed):
+    """FP8 attention on random lengths (around every tile boundary, query and key lengths unequal), both layouts and
+    dtypes, every combination of scale recipe, probability rule and K block, inputs with and without outliers and with
+    rising row maxima: against the oracle that re-quantises the probabilities the way the kernel does."""
+    from mindiesd.layers.quant import fp8_attention_forward
+    from oracle import quant as oq
+    r = random.Random(700 + seed)
+    dtype, layout = r.choice([torch.bfloat16, torch.float16]), r.choice(["BNSD", "BSND"])
+    sq, skv, n = r.choice(SQ), r.choice([s for s in SKV if s >= 3]), r.choice([1, 2, 3])
+    recipe, p_rule, k_block = r.choice(["amax", "pow2"]), r.choice(["linear", "exp2"]), r.choice([128, 256])
+    g = torch.Generator().manual_seed(seed)
+    def make(s):
+        x = torch.randn((1, n, s, 128), generator=g)
+        if seed % 3:
+            x = torch.where(torch.rand((1, n, s, 128), generator=g) < 0.01, x * 8, x)
+        return x.to(dtype)
+    q, k, v = make(sq), make(skv), make(skv)
+    if seed % 2:
+        k[:, :, skv // 2:] *= 1.7                      # the reference maximum has to move late in the row
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True, p_rule=p_rule, k_block=k_block).float()
+    args = (q, k, v) if layout == "BNSD" else tuple(t.transpose(1, 2).contiguous() for t in (q, k, v))
+    out = fp8_attention_forward(*(t.to(cuda) for t in args), layout=layout, recipe=recipe, p_rule=p_rule,
+                                k_block=k_block).cpu().float()
+    out = out if layout == "BNSD" else out.transpose(1, 2)
+    case = (dtype, layout, sq, skv, n, recipe, p_rule, k_block)
+    assert bool(torch.isfinite(out).all()), case
+    err = (out - want).abs().max().item()
+    assert oa.cosine(out, want) >= 0.9999 and err <= 2.0 ** -5 * max(1.0, want.abs().max().item()), (case, err)
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_varlen_random_sequences(cuda, seed):
     import mindiesd
