@@ -164,8 +164,10 @@ __global__ __launch_bounds__(256) void block_quant128_kernel(const void* x_, uns
 // One workgroup = one 128-token block; R^T sits in LDS (16-byte chunk c of row n at chunk c ^ (n & 15)); wave w
 // owns tokens 32w..32w+31.  R^T is the first matrix operand, so a lane holds one token and, per register
 // quad, four consecutive output channels = one dword of codes.
+// (launch bounds: at least 4 waves per SIMD = 128 registers per lane, so that the four workgroups whose LDS fits a CU
+// are resident together - the pass is bound by memory latency)
 template <int DT>
-__global__ __launch_bounds__(256) void rot_block_quant_kernel(const void* x_, const void* rot_t_, unsigned char* q,
+__global__ __launch_bounds__(256, 4) void rot_block_quant_kernel(const void* x_, const void* rot_t_, unsigned char* q,
                                                               float* scale, long long sb, long long sn, long long ss,
                                                               int N, int S, float prescale, int pow2) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -222,16 +224,29 @@ __global__ __launch_bounds__(256) void rot_block_quant_kernel(const void* x_, co
   amax = block_max_256(amax, red);
   const float sc = block_scale(amax, pow2);
   if (tid == 0) scale[(long long)bn * nblk + blk] = sc;
-  if (ok) {
-    unsigned char* qo = q + ((long long)bn * S + tok) * 128;
+  // The codes of a token (128 bytes) are spread over the lanes in dwords; they go through LDS (R^T is no longer
+  // needed: block_max_256 has synchronised the workgroup after the last matrix instruction) so that the stores to
+  // global memory are whole 16-byte chunks of consecutive rows.  16-byte chunk c of token row r sits at chunk
+  // c ^ (r & 7).
+  {
+    const int r = wave * 32 + l32;
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int w = pack4_e4m3(__fdiv_rn(acc[nb][4 * g], sc), __fdiv_rn(acc[nb][4 * g + 1], sc),
                                  __fdiv_rn(acc[nb][4 * g + 2], sc), __fdiv_rn(acc[nb][4 * g + 3], sc));
-        *(int*)(qo + nb * 32 + 8 * g + 4 * h) = w;
+        const int byte = nb * 32 + 8 * g + 4 * h;
+        *(int*)(rt_lds + r * 128 + (((byte >> 4) ^ (r & 7)) << 4) + (byte & 15)) = w;
       }
+  }
+  __syncthreads();
+  unsigned char* qo = q + ((long long)bn * S + row0) * 128;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tid >> 3) + 32 * i, c = tid & 7;
+    const i32x4_t w = *(const i32x4_t*)(rt_lds + r * 128 + ((c ^ (r & 7)) << 4));
+    if (row0 + r < S) *(i32x4_t*)(qo + (long long)r * 128 + c * 16) = w;
   }
 #endif
 }
@@ -752,7 +767,7 @@ int mindiesd_fa_rot_block_quant(const void* x, const void* rot_t, void* q, float
   if (!x || !rot_t || !q || !scale || B <= 0 || N <= 0 || S <= 0 || !(prescale > 0.f)) return MSD_ERR_BAD_ARG;
   if (D != 128) return MSD_ERR_UNSUPPORTED;
   if (dtype != MSD_DTYPE_BF16 && dtype != MSD_DTYPE_F16) return MSD_ERR_BAD_ARG;
-  if ((((uintptr_t)x | (uintptr_t)rot_t) & 15) || ((uintptr_t)q & 3) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
+  if ((((uintptr_t)x | (uintptr_t)rot_t) & 15) || ((uintptr_t)q & 15) || ((x_sb | x_sn | x_ss) & 7)) return MSD_ERR_BAD_ARG;
   const dim3 grid((S + 127) / 128, B * N);
   if (grid.y > 65535) return MSD_ERR_UNSUPPORTED;
   if (dtype == MSD_DTYPE_BF16)
