@@ -44,4 +44,9 @@ struct FaParams {
 // the general mode (packed sequences, causal, boolean mask, lse).
 int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream);
 
+// Dense attention at head_dim 64 exactly (flash_attn_d64.hip): no mask, no packed sequences; `supported` is false when
+// a K or V (batch, head) slice does not fit the kernel's 32-bit buffer offsets (the general kernel takes those).
+bool fa16_d64_supported(const FaParams& p);
+int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream);
+
 }  // namespace msd

@@ -1113,6 +1113,7 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale, true);
   if (rc != MSD_OK) return rc;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
+  if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream);
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16>(p, stream);
   return launch_fa16<MSD_DTYPE_F16>(p, stream);

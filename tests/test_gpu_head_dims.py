@@ -111,6 +111,27 @@ def test_varlen(cuda, d, causal):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sq,skv", [(2311, 3001), (256, 128), (257, 129), (33, 4100)])
+def test_head_dim_64_dense_kernel_against_general_kernel_and_oracle(cuda, sq, skv, dtype):
+    """Dense head_dim 64 without a mask runs on its own kernel (csrc/flash_attn_d64.hip); an all-true mask sends the
+    same inputs through the general kernel.  Query and key lengths off every tile boundary, grouped-query heads,
+    BSND storage; sampled rows against the oracle, everything (and the log-sum-exp) against the general kernel."""
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    q, k, v = _rand((1, sq, 6, 64), 50, dtype), _rand((1, skv, 2, 64), 51, dtype), _rand((1, skv, 2, 64), 52, dtype)
+    dq, dk, dv = q.to(cuda), k.to(cuda), v.to(cuda)
+    out, lse = flash_attention(dq, dk, dv, 0.125, "BSND", return_lse=True)
+    gen, lse_g = flash_attention(dq, dk, dv, 0.125, "BSND", return_lse=True,
+                                 attn_mask=torch.ones(sq, skv, dtype=torch.bool, device=cuda))
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3
+    assert (out.float() - gen.float()).abs().max().item() <= tol
+    assert (lse - lse_g).abs().max().item() < 1e-3
+    rows = sorted({0, 1, 15, 16, 31, 32, sq // 2, sq - 2, sq - 1} & set(range(sq)))
+    kk, vv = k.repeat_interleave(3, dim=2), v.repeat_interleave(3, dim=2)
+    ref = attention_math(q[:, rows], kk, vv, None, 0.125, head_first=False)
+    _check(out[:, rows].cpu(), ref, max_abs=tol, min_cos=0.9999 if dtype == torch.bfloat16 else 0.99999)
+
+
 def test_rejected_head_dims(cuda):
     import mindiesd
     from mindiesd.utils.exception import ParametersInvalid
