@@ -178,7 +178,8 @@ def extra_dense_1p3b(device, steps, warmup):
 
 
 def extra_head_dims(device, steps, warmup):
-    """Dense attention at head dims other than 128 (the generic kernel): 64 and 256 at a 17776-token sequence."""
+    """Dense attention at head dims other than 128 at a 17776-token sequence: 64 (its own kernel) and 256 (the general
+    kernel)."""
     import torch
     import mindiesd
     res = {"workload": "dense bf16 B1 S17776 (13x30x45 latent tokens + 226 text tokens), N48 D64 / N12 D256"}
@@ -189,6 +190,7 @@ def extra_head_dims(device, steps, warmup):
         m = median(ms)
         res[f"d{d}_ms"] = m
         res[f"d{d}_tflops"] = 4.0 * n * 17776 * 17776 * d / m / 1e9
+        res[f"d{d}_frac_of_bf16_peak"] = res[f"d{d}_tflops"] / PEAK_BF16_TFLOPS
     return res
 
 
