@@ -208,12 +208,20 @@ def extra_causal_varlen(device, steps, warmup):
     cu = torch.tensor([0] + lens).cumsum(0).tolist()
     qt, kt, vt = (t[0].transpose(0, 1).contiguous() for t in (q, k, v))
     v_ms, _ = time_steps(lambda: mindiesd.attention_forward_varlen(qt, kt, vt, cu, cu), steps, warmup)
+    # boolean masks, all true (timing of the mask path itself): one row shared by all queries, and a full [S, S] one
+    pad = torch.ones(1, 1, 1, s, dtype=torch.bool, device=device).expand(1, 1, s, s)
+    p_ms, _ = time_steps(lambda: flash_attention(q, k, v, d ** -0.5, "BNSD", attn_mask=pad), steps, warmup)
+    full = torch.ones(s, s, dtype=torch.bool, device=device)
+    f_ms, _ = time_steps(lambda: flash_attention(q, k, v, d ** -0.5, "BNSD", attn_mask=full), steps, warmup)
+    del full
     cm, vm = median(c_ms), median(v_ms)
     causal_flops = 4.0 * n * d * (s * (s + 1) / 2)
     varlen_flops = 4.0 * n * d * sum(l * l for l in lens)
     return {"workload": "bf16 B1 N12 S32760 D128: causal; and packed as 7 sequences " + str(lens),
             "causal_ms": cm, "causal_tflops_unmasked_work": causal_flops / cm / 1e9,
-            "varlen_ms": vm, "varlen_tflops": varlen_flops / vm / 1e9}
+            "varlen_ms": vm, "varlen_tflops": varlen_flops / vm / 1e9,
+            "key_padding_mask_ms": median(p_ms), "full_mask_ms": median(f_ms),
+            "full_mask_tflops": attn_flops(cfg) / median(f_ms) / 1e9}
 
 
 def extra_sparse(device, steps, warmup, dense_ms):

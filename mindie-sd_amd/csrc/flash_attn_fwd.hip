@@ -307,6 +307,23 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int dense_tiles = (kv_lim + BN - 1) / BN;
   const unsigned char* mask_g = nullptr;
   if (MODE && p.mask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
+  // Boolean mask of a tile that lies wholly inside the sequence: the lane fetches the BN bytes of its own query row as
+  // 16-byte words (any alignment: global loads take unaligned addresses) one tile ahead, into the set that belongs to
+  // the tile's LDS stage, so they arrive with the tile's own data and cost no wait of their own.  The tile that runs
+  // past the end of the row is tested byte by byte instead (a 16-byte read could leave the mask there).
+  i32x4_t mask_w[2][C::kNQB][C::kNKB][2];
+  auto mask_fetch = [&](int key0, auto stage_c) __attribute__((always_inline)) {
+    constexpr int st = decltype(stage_c)::value;
+#pragma unroll
+    for (int qb = 0; qb < C::kNQB; ++qb) {
+      const int qrow = min(q0 + wave * QPW + qb * 32 + l32, Sq - 1);
+      const unsigned char* mrow = mask_g + (long long)qrow * p.m_sq + key0;
+#pragma unroll
+      for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) __builtin_memcpy(&mask_w[st][qb][kb][hf], mrow + kb * 32 + 16 * hf, 16);
+    }
+  };
   auto stream_next = [&](int& key0, int& fl) {  // sparse: produce the tile after the one produced last
     if (sub > 0) {  // remaining sub-tiles of the current 128-key block
       key0 = key0 + BN;
@@ -336,6 +353,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
   } else {
     load_tile(0, 0);
+    if (MODE && mask_g && BN <= Skv) mask_fetch(0, std::integral_constant<int, 0>{});
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
@@ -350,6 +368,8 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   auto tile_step = [&](auto stage_c, const int key0, const int next_key0, const bool active) {
     constexpr int stage = decltype(stage_c)::value;
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+    if (MODE && !SPARSE && mask_g && next_key0 >= 0 && next_key0 + BN <= Skv)
+      mask_fetch(next_key0, std::integral_constant<int, stage ^ 1>{});
     if (active) {
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
     MSD_LDS const char* vb_base = kb_base + C::kTileBytes;
@@ -415,7 +435,21 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         }
       }
       // boolean mask: one byte per (query, key); a lane tests the 16 x kNKB keys of its own query row
-      if (mask_g) {
+      if (mask_g && !SPARSE && key0 + BN <= Skv) {
+        // register r of block kb is key 32 kb + 8 (r / 4) + 4 h + r % 4: dword 2 (r / 4) + h of the block's 32 bytes
+#pragma unroll
+        for (int qb = 0; qb < C::kNQB; ++qb)
+#pragma unroll
+          for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const i32x4_t w4 = mask_w[stage][qb][kb][g4 >> 1];
+              const unsigned w = (unsigned)(h ? w4[2 * (g4 & 1) + 1] : w4[2 * (g4 & 1)]);
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (((w >> (8 * j)) & 0xffu) == 0) sacc[kb][qb][4 * g4 + j] = -INFINITY;
+            }
+      } else if (mask_g) {
 #pragma unroll
         for (int qb = 0; qb < C::kNQB; ++qb) {
           const int qrow = min(q0 + wave * QPW + qb * 32 + l32, Sq - 1);

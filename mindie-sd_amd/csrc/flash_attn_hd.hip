@@ -150,7 +150,24 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   // 4*(lane%4) of a 32-wide block
   const int v_off = (4 * h + ((lane & 15) >> 2)) * C::kRowBytes + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
 
+  // Boolean mask of a tile that lies wholly inside the sequence: the lane fetches the bytes of its own query row that
+  // belong to its score registers as 4-byte words (register r of block kb is key 32 kb + 8 (r / 4) + 4 h + r % 4: one
+  // word per r / 4; any alignment - global loads take unaligned addresses), one tile ahead.  With a mask the K/V
+  // chunks of the next tile are requested after the mask test instead of at the top of the step, so that the words
+  // are never waited for with younger requests in flight.  The tile that runs past the end of the row is tested byte
+  // by byte instead (a 4-byte read could leave the mask there).
+  unsigned mask_w[C::kNKB][4];
+  auto mask_fetch = [&](int key0) __attribute__((always_inline)) {
+    const int qrow = min(q0 + wave * 32 + l32, Sq - 1);
+    const unsigned char* mrow = mask_g + (long long)qrow * p.m_sq + key0 + 4 * h;
+#pragma unroll
+    for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) __builtin_memcpy(&mask_w[kb][g4], mrow + kb * 32 + 8 * g4, 4);
+  };
+
   if (tiles > 0) {
+    if (mask_g && C::kBN <= Skv) mask_fetch(0);
     fetch(0);
     stash(0);
   }
@@ -159,7 +176,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   for (int t = 0; t < tiles; ++t) {
     const int stage = t & 1;
     const int key0 = t * C::kBN;
-    if (t + 1 < tiles) fetch(key0 + C::kBN);
+    if (!mask_g && t + 1 < tiles) fetch(key0 + C::kBN);
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
     MSD_LDS const char* vb_base = kb_base + C::kTileBytes;
 
@@ -177,9 +194,20 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
     const int qrow = q0 + wave * 32 + l32;
     const bool edge = key0 + C::kBN > Skv;
     const bool diag = p.causal && key0 + C::kBN - 1 > q0 + wave * 32 + causal_shift;
-    if (edge || diag || mask_g) {
+    if (mask_g && !edge) {
+#pragma unroll
+      for (int kb = 0; kb < C::kNKB; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (((mask_w[kb][r >> 2] >> (8 * (r & 3))) & 0xffu) == 0) sacc[kb][r] = -INFINITY;
+    }
+    if (mask_g && t + 1 < tiles) {
+      if (key0 + 2 * C::kBN <= Skv) mask_fetch(key0 + C::kBN);
+      fetch(key0 + C::kBN);
+    }
+    if (edge || diag) {
       const int last_visible = p.causal ? qrow + causal_shift : 0x7fffffff;
-      const unsigned char* mrow = mask_g ? mask_g + (long long)min(qrow, Sq - 1) * p.m_sq : nullptr;
+      const unsigned char* mrow = (mask_g && edge) ? mask_g + (long long)min(qrow, Sq - 1) * p.m_sq : nullptr;
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
