@@ -360,15 +360,26 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
   auto write_tile = [&](auto bias_c) {
     constexpr bool BIAS = decltype(bias_c)::value;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int nb = 0; nb < 2; ++nb) {
+      // the bias of this block's columns, fetched once for all rows (columns past the end read column 0: never stored)
+      f32x4_t bias_r[2][4];  // [w][j]; SwiGLU: w = 0 gate, w = 1 up
+      if (BIAS) {
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const int m = m0 + a * 128 + wm * 64 + mb * 32 + l32;
-        T* orow = og + (long long)m * p.Nout;
+        for (int w = 0; w < 2; ++w)
 #pragma unroll
-        for (int w = 0; w < (SWIGLU ? 1 : 2); ++w)
+          for (int j = 0; j < 4; ++j) {
+            const int col = f0 + (SWIGLU ? 0 : w * 128) + wn * 64 + nb * 32 + 8 * j + 4 * h;
+            bias_r[w][j] = *(const f32x4_t*)(p.bias + (SWIGLU ? w * half : 0) + (col < p.Nout ? col : 0));
+          }
+      }
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb)
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+          const int m = m0 + a * 128 + wm * 64 + mb * 32 + l32;
+          T* orow = og + (long long)m * p.Nout;
+#pragma unroll
+          for (int w = 0; w < (SWIGLU ? 1 : 2); ++w)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const int ncol = wn * 64 + nb * 32 + 8 * j + 4 * h;  // first of the four columns, tile-local
@@ -377,9 +388,9 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
               float v[4];
               if (SWIGLU) {
                 f32x4_t bg = {0.f, 0.f, 0.f, 0.f}, bu = {0.f, 0.f, 0.f, 0.f};
-                if (BIAS) {  // columns past the end read column 0 (never stored)
-                  bg = *(const f32x4_t*)(p.bias + (col_ok ? col : 0));
-                  bu = *(const f32x4_t*)(p.bias + half + (col_ok ? col : 0));
+                if (BIAS) {
+                  bg = bias_r[0][j];
+                  bu = bias_r[1][j];
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -389,7 +400,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
                 }
               } else {
                 f32x4_t bv = {0.f, 0.f, 0.f, 0.f};
-                if (BIAS) bv = *(const f32x4_t*)(p.bias + (col_ok ? col : 0));
+                if (BIAS) bv = bias_r[w][j];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = acc[a][w][mb][nb][4 * j + e] + bv[e];
               }
@@ -398,7 +409,8 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_kernel(const GemmParams p) 
                 *(i32x2_t*)(orow + col) = *(const i32x2_t*)t4;
               }
             }
-      }
+        }
+    }
   };
   if (p.bias) write_tile(std::true_type{});
   else write_tile(std::false_type{});
