@@ -194,6 +194,27 @@ def extra_head_dims(device, steps, warmup):
     return res
 
 
+def extra_cross_attention(device, steps, warmup):
+    """Dense attention of the 720p video tokens over a short text (few key tiles per query tile: the launch is
+    mostly reading Q and writing O)."""
+    import torch
+    import mindiesd
+    cfg = CFG_14B_720P
+    n, s, d = cfg["N"], cfg["S"], cfg["D"]
+    g = torch.Generator(device=device).manual_seed(11)
+    q = (torch.randn((1, n, s, d), device=device, generator=g) * 0.5).to(torch.bfloat16)
+    res = {"workload": f"dense bf16 B1 N{n} Sq{s} D{d} over 226 / 512 keys",
+           "q_plus_out_gb": 2.0 * n * s * d * 2 / 1e9}
+    for skv in (226, 512):
+        k, v = ((torch.randn((1, n, skv, d), device=device, generator=g) * 0.5).to(torch.bfloat16) for _ in range(2))
+        ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)
+        m = median(ms)
+        res[f"skv{skv}_ms"] = m
+        res[f"skv{skv}_tflops"] = 4.0 * n * s * skv * d / m / 1e9
+        res[f"skv{skv}_frac_of_hbm_peak"] = res["q_plus_out_gb"] / m * 1e3 / PEAK_HBM_GBS
+    return res
+
+
 def extra_causal_varlen(device, steps, warmup):
     """General mode of the dense kernel at the 1.3B shape: bottom-right causal mask (about half of the
     score matrix is skipped) and the same tokens packed as 7 sequences of unequal length."""
@@ -421,7 +442,7 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference kernel for scaling rocprof byte counters)")
     ap.add_argument("--extras-only", default="",
-                    help="comma separated subset of extras to run (dense_wan1p3b,causal_varlen,sparse_rf_v3,ada_bsa,fp8_attention,"
+                    help="comma separated subset of extras to run (dense_wan1p3b,head_dims,cross_attention,causal_varlen,sparse_rf_v3,ada_bsa,fp8_attention,"
                          "mxfp8_gemm_swiglu)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -477,6 +498,7 @@ def main():
         extras = {}
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
                          ("head_dims", lambda: extra_head_dims(device, args.steps, args.warmup)),
+                         ("cross_attention", lambda: extra_cross_attention(device, args.steps, args.warmup)),
                          ("causal_varlen", lambda: extra_causal_varlen(device, args.steps, args.warmup)),
                          ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
                          ("ada_bsa", lambda: extra_ada_bsa(device, args.steps, args.warmup, kernel_ms)),
