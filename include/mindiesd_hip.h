@@ -74,6 +74,28 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
                                          const unsigned char* mask, long long m_sb, long long m_sn, long long m_sq,
                                          hipStream_t stream);
 
+/* Packed sequences whose lengths only the device knows (cu_seqlens given as device tensors to
+ * attention_forward_varlen, mindiesd/layers/flash_attn/attention_forward_varlen.py:45-149; the reference hands
+ * them to torch_npu.npu_fusion_attention as actual_seq_qlen / actual_seq_kvlen, :141-149): q, out
+ * [total_q][N][D], k, v [total_k][Nkv][D] with element strides of head and token, seq_meta int32 [B][4] as in
+ * mindiesd_flash_attention_general_fwd.  The grid is sized from the token totals (at most ceil(total_q / 128) + B
+ * query tiles per head exist whatever the lengths are) and every workgroup finds its sequence in the table; the
+ * general entry point with Sq = total_q as the only bound launches B times as many.  The query counts of the table
+ * must not add up to more than total_q: tiles beyond the bound are not computed.  causal as above. */
+int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void* v, void* out, int dtype,
+                                        int B, int N, int Nkv, int total_q, int total_k, int D,
+                                        long long q_sn, long long q_ss, long long k_sn, long long k_ss,
+                                        long long v_sn, long long v_ss, long long o_sn, long long o_ss,
+                                        float scale, const int* seq_meta, int causal, hipStream_t stream);
+
+/* cu_seqlens_q / cu_seqlens_k as attention_forward_varlen receives them (device arrays, int32, B + 1 entries each;
+ * mindiesd/layers/flash_attn/attention_forward_varlen.py:86-89) -> the seq_meta table [B][4] of the two entry points
+ * above, built on the device without a host read-back: first tokens are clamped to [0, total], counts to what lies
+ * behind them and to max_q / max_k (pass the token totals when the longest sequence is not known).  seq_meta must be
+ * 16-byte aligned. */
+int mindiesd_varlen_meta(const int* cu_seqlens_q, const int* cu_seqlens_k, int B, int total_q, int total_k,
+                         int max_q, int max_k, int* seq_meta, hipStream_t stream);
+
 /* ---- block-sparse attention ------------------------------------------------------------------------
  * Query block i (128 rows) of (b, n) attends to the 128-key blocks blk_idx[b][n][i][0 .. blk_cnt[b][n][i])
  * (ascending ids, int32, row pitch kb_stride); an empty list gives zeros.  `order` (optional,

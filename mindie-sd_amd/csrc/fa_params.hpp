@@ -34,11 +34,45 @@ struct FaParams {
   // general mode (MODE = 1 instantiations only)
   const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
                               // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count
+  int packed_tiles;           // > 0 (with seq_meta): the grid holds this many 128-row query tiles per head, numbered
+                              // through the sequences (tile i belongs to the sequence the running sum of
+                              // ceil(query count / 128) reaches it in); 0: B x ceil(Sq / 128) tiles per head
   int lse_token_major;        // with seq_meta: lse is [tokens][N] (index (first query token + row) * N + head)
   int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
   const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
   long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
 };
+
+#if defined(__HIP_DEVICE_COMPILE__)
+// Packed numbering of the query tiles (FaParams::packed_tiles): which sequence tile i of a head belongs to and which
+// of that sequence's 128-row tiles it is.  Every lane of the wave takes one sequence of a group of 64, the running
+// sum of the tile counts is a wave scan; the result is wave-uniform.  False: i lies past the last tile.
+__device__ __forceinline__ bool packed_find_tile(const int* seq_meta, int nseq, int i, int& seq, int& tile) {
+  const int lane = threadIdx.x & 63;
+  int base = 0;
+  for (int c0 = 0; c0 < nseq; c0 += 64) {
+    const int s = c0 + lane;
+    const int t = s < nseq ? (seq_meta[4 * s + 1] + 127) / 128 : 0;
+    int incl = t;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int u = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += u;
+    }
+    const int total = __shfl(incl, 63, 64);
+    if (i < base + total) {
+      const int first = base + incl - t;
+      const unsigned long long hit = __ballot(t > 0 && i >= first && i < first + t);
+      const int l = __ffsll((long long)hit) - 1;  // exactly one lane holds tile i
+      seq = c0 + l;
+      tile = i - __shfl(first, l, 64);
+      return true;
+    }
+    base += total;
+  }
+  return false;
+}
+#endif
 
 // Dense attention for head dims other than 128 (flash_attn_hd.hip): D a multiple of 8, at most 256; all options of
 // the general mode (packed sequences, causal, boolean mask, lse).

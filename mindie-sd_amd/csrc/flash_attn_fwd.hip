@@ -114,8 +114,9 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int h = lane >> 5;
 
   // ---- which (batch, head, query tile): consecutive tiles of one head stay on one XCD -------
-  const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
-  const int total = p.B * p.N * q_tiles;
+  const bool packed = MODE && !SPARSE && p.packed_tiles > 0;
+  const int q_tiles = packed ? p.packed_tiles : (p.Sq + C::kBM - 1) / C::kBM;
+  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
   int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (SPARSE && p.order) {  // caller's work order: workgroup i takes entry i of the table
@@ -123,11 +124,20 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     work = p.order[blockIdx.x];
   }
   if (work < 0 || work >= total) return;
-  const int bn = work / q_tiles;
+  int bn = work / q_tiles;
   int qt = work - bn * q_tiles;
-  if (MODE && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
-  const int b = bn / p.N;
-  const int n = bn - b * p.N;
+  int b, n;
+  if (packed) {  // bn is the head; the tile's sequence comes from the table (kBM = 128 here)
+    static_assert(!MODE || SPARSE || C::kBM == 128, "packed numbering counts 128-row tiles");
+    n = bn;
+    if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt)) return;
+    if (p.causal) qt = (p.seq_meta[4 * b + 1] + C::kBM - 1) / C::kBM - 1 - qt;
+    bn = b * p.N + n;
+  } else {
+    if (MODE && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
+    b = bn / p.N;
+    n = bn - b * p.N;
+  }
   const int nkv = n / (p.N / p.Nkv);
   const int q0 = qt * C::kBM;
 
@@ -1000,10 +1010,23 @@ static int launch_fa(const FaParams& p, hipStream_t stream) {
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
     return MSD_ERR_LAUNCH;
   const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
-  const int total = p.B * p.N * q_tiles;
+  const int total = (MODE && !SPARSE && p.packed_tiles > 0) ? p.N * p.packed_tiles : p.B * p.N * q_tiles;
   const int grid = ((total + 7) / 8) * 8;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kNT), C::kLdsBytes, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+
+
+// cumulative lengths (device) -> the [B][4] table of the packed / general entry points, clamped to the tensors
+__global__ void varlen_meta_kernel(const int* cu_q, const int* cu_k, int B, int total_q, int total_k, int max_q,
+                                   int max_k, int* meta) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  const int q0 = min(max(cu_q[b], 0), total_q), k0 = min(max(cu_k[b], 0), total_k);
+  const int lq = min(min(max(cu_q[b + 1] - cu_q[b], 0), total_q - q0), max_q);
+  const int lk = min(min(max(cu_k[b + 1] - cu_k[b], 0), total_k - k0), max_k);
+  *(i32x4_t*)(meta + 4 * b) = i32x4_t{q0, lq, k0, lk};
 }
 
 }  // namespace msd
@@ -1231,6 +1254,44 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
+  if (D != 128) return launch_fa_hd(p, dtype, D, stream);
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
+}
+
+// cu_seqlens_q / cu_seqlens_k (device, int32, B + 1 entries each) -> seq_meta [B][4] for the two entry points that
+// take it, without a host read-back: first tokens clamped to the tensors, counts to what is left behind them and to
+// max_q / max_k (pass the token totals when the longest sequence is not known).
+int mindiesd_varlen_meta(const int* cu_seqlens_q, const int* cu_seqlens_k, int B, int total_q, int total_k, int max_q,
+                         int max_k, int* seq_meta, hipStream_t stream) {
+  if (!cu_seqlens_q || !cu_seqlens_k || !seq_meta || B <= 0 || total_q < 0 || total_k < 0 || max_q < 0 || max_k < 0)
+    return MSD_ERR_BAD_ARG;
+  if ((uintptr_t)seq_meta & 15) return MSD_ERR_BAD_ARG;
+  hipLaunchKernelGGL(varlen_meta_kernel, dim3((B + 255) / 256), dim3(256), 0, stream, cu_seqlens_q, cu_seqlens_k, B,
+                     total_q, total_k, max_q, max_k, seq_meta);
+  return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+// Packed sequences whose lengths only the device knows: q, out [total_q][N][D], k, v [total_k][Nkv][D] (token, head
+// strides), seq_meta as above with B sequences.  The grid is sized from the token total - at most
+// ceil(total_q / 128) + B query tiles per head exist whatever the lengths are - and every workgroup looks its
+// sequence up in the table, where mindiesd_flash_attention_general_fwd with Sq = total_q as the only known bound
+// launches B x ceil(total_q / 128) workgroups per head, nearly all of which return at once.  The query counts of the
+// table must not add up to more than total_q (tiles beyond the bound are not computed).
+int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void* v, void* out, int dtype, int B, int N,
+                                        int Nkv, int total_q, int total_k, int D, long long q_sn, long long q_ss,
+                                        long long k_sn, long long k_ss, long long v_sn, long long v_ss, long long o_sn,
+                                        long long o_ss, float scale, const int* seq_meta, int causal,
+                                        hipStream_t stream) {
+  const long long st[12] = {0, q_sn, q_ss, 0, k_sn, k_ss, 0, v_sn, v_ss, 0, o_sn, o_ss};
+  const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, total_q, total_k, D, st, scale, true);
+  if (rc != MSD_OK) return rc;
+  if (!seq_meta) return MSD_ERR_BAD_ARG;
+  FaParams p = make_params(q, k, v, out, nullptr, B, N, Nkv, total_q, total_k, st, scale);
+  p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
+  const long long tiles = ((long long)total_q + 127) / 128 + B;
+  if (tiles * N > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
+  p.packed_tiles = (int)tiles;
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);

@@ -57,16 +57,25 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   const int h = lane >> 5;
 
   // consecutive query tiles of one head stay on one XCD (workgroups are dealt round-robin to the 8 XCDs)
-  const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
-  const int total = p.B * p.N * q_tiles;
+  const bool packed = p.packed_tiles > 0;  // the tiles of a head are numbered through the packed sequences
+  const int q_tiles = packed ? p.packed_tiles : (p.Sq + C::kBM - 1) / C::kBM;
+  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
   const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
   const int bn = work / q_tiles;
   int qt = work - bn * q_tiles;
-  if (p.causal) qt = q_tiles - 1 - qt;
-  const int b = bn / p.N;
-  const int n = bn - b * p.N;
+  int b, n;
+  if (packed) {
+    static_assert(C::kBM == 128, "packed numbering counts 128-row tiles");
+    n = bn;
+    if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt)) return;
+    if (p.causal) qt = (p.seq_meta[4 * b + 1] + C::kBM - 1) / C::kBM - 1 - qt;
+  } else {
+    if (p.causal) qt = q_tiles - 1 - qt;
+    b = bn / p.N;
+    n = bn - b * p.N;
+  }
   const int nkv = n / (p.N / p.Nkv);
   const int q0 = qt * C::kBM;
 
@@ -324,7 +333,8 @@ static int launch_hd(const FaParams& p, int D, hipStream_t stream) {
   auto kern = fa_hd_kernel<DT, DP>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const long long total = (long long)p.B * p.N * ((p.Sq + C::kBM - 1) / C::kBM);
+  const long long total = p.packed_tiles > 0 ? (long long)p.N * p.packed_tiles
+                                             : (long long)p.B * p.N * ((p.Sq + C::kBM - 1) / C::kBM);
   if (total > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kern, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), C::kLds, stream, p, D);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;

@@ -25,6 +25,8 @@ c_int, c_ll, c_f, c_p, c_sz = ctypes.c_int, ctypes.c_longlong, ctypes.c_float, c
 SIGNATURES = {
     "mindiesd_flash_attention_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p]),
     "mindiesd_flash_attention_general_fwd": (c_int, [c_p] * 5 + [c_int] * 7 + [c_ll] * 12 + [c_f, c_p, c_int, c_p] + [c_ll] * 3 + [c_p]),
+    "mindiesd_flash_attention_packed_fwd": (c_int, [c_p] * 4 + [c_int] * 7 + [c_ll] * 8 + [c_f, c_p, c_int, c_p]),
+    "mindiesd_varlen_meta": (c_int, [c_p] * 2 + [c_int] * 5 + [c_p] * 2),
     "mindiesd_ada_block_sparse_attention_fwd": (c_int, [c_p] * 4 + [c_int] * 6 + [c_ll] * 12 + [c_f, c_p, c_p, c_int, c_int, c_p]),
     "mindiesd_sbe_scores_workspace_size": (c_sz, [c_int, c_int]),
     "mindiesd_sbe_scores": (c_int, [c_p, c_p, c_p] + [c_int] * 6 + [c_ll] * 6 + [c_f, c_int, c_p, c_sz, c_p]),

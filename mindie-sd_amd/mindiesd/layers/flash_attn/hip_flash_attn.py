@@ -108,17 +108,15 @@ def _varlen_meta(cu_q, cu_k, total_q, total_k, device, max_q=None, max_k=None):
     if on_device:
         if cu_q.dim() != 1 or cu_k.dim() != 1 or cu_q.shape[0] != cu_k.shape[0] or cu_q.shape[0] < 2:
             raise ParametersInvalid("cu_seqlens_q and cu_seqlens_k must be 1-D with batch_size + 1 entries each.")
-        cq, ck = cu_q.to(device=device, dtype=torch.int64), cu_k.to(device=device, dtype=torch.int64)
-        sq0, sk0 = cq[:-1].clamp(0, total_q), ck[:-1].clamp(0, total_k)
-        lq = (cq[1:] - cq[:-1]).clamp(min=0)
-        lk = (ck[1:] - ck[:-1]).clamp(min=0)
-        lq, lk = torch.minimum(lq, total_q - sq0), torch.minimum(lk, total_k - sk0)
-        meta = torch.stack([sq0, lq, sk0, lk], dim=1).to(torch.int32).contiguous()
+        cq = cu_q.to(device=device, dtype=torch.int32).contiguous()   # no copies when they already are int32
+        ck = cu_k.to(device=device, dtype=torch.int32).contiguous()
         bound_q = total_q if max_q is None else max(min(int(max_q), total_q), 1)
-        bound_k = total_k if max_k is None else min(int(max_k), total_k)
-        if max_q is not None or max_k is not None:   # the named bounds hold whatever the table says
-            meta = torch.stack([sq0, lq.clamp(max=bound_q), sk0, lk.clamp(max=max(bound_k, 0))], dim=1) \
-                .to(torch.int32).contiguous()
+        bound_k = total_k if max_k is None else max(min(int(max_k), total_k), 0)
+        meta = torch.empty((cq.shape[0] - 1, 4), dtype=torch.int32, device=device)
+        with torch.cuda.device(device):
+            rc = _native.lib().mindiesd_varlen_meta(cq.data_ptr(), ck.data_ptr(), cq.shape[0] - 1, total_q, total_k,
+                                                    bound_q, bound_k, meta.data_ptr(), _native.stream_ptr(device))
+        _native.check(rc, "mindiesd_varlen_meta")
         return meta, bound_q, max(bound_k, 1), cq.shape[0] - 1
     def lengths(cu, name):
         vals = [int(x) for x in (cu.detach().cpu().tolist() if isinstance(cu, torch.Tensor) else cu)]
@@ -161,6 +159,16 @@ def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=Fa
     if max_q == 0:
         return out
     tn = lambda t: (0, t.stride(1), t.stride(0))  # (batch, head, token) strides of a [T, N, D] tensor
+    if unchecked and max_seqlen_q is None and max_seqlen_k is None:
+        # lengths known to the device only: the grid comes from the token totals, the workgroups find their sequence
+        with torch.cuda.device(q.device):
+            rc = _native.lib().mindiesd_flash_attention_packed_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _native.DTYPE_CODE[q.dtype],
+                nseq, q.shape[1], k.shape[1], q.shape[0], k.shape[0], q.shape[2],
+                *tn(q)[1:], *tn(k)[1:], *tn(v)[1:], *tn(out)[1:], float(scale), meta_t.data_ptr(), int(bool(causal)),
+                _native.stream_ptr(q.device))
+        _native.check(rc, "mindiesd_flash_attention_packed_fwd")
+        return out
     with torch.cuda.device(q.device):
         rc = _native.lib().mindiesd_flash_attention_general_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None, _native.DTYPE_CODE[q.dtype],

@@ -127,6 +127,27 @@ def test_varlen_device_table_uncovered_rows_and_named_bounds(cuda):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_many_sequences_device_table(cuda, d, causal):
+    """150 sequences (more than one wave's worth of table entries) of lengths 0 .. 300, key lengths different from the
+    query lengths, cu_seqlens on the device: the packed entry point numbers the query tiles through the sequences.
+    Same result as with the host lists (which size the grid by the longest sequence) and parity with the oracle."""
+    import random
+    import mindiesd
+    r = random.Random(d + causal)
+    lens_q = [r.choice([0, 1, 5, 127, 128, 129, 200, 300]) for _ in range(150)]
+    lens_k = [max(1, l + r.choice([-3, 0, 0, 40])) for l in lens_q]
+    cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+    cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+    q, k, v = _rand((sum(lens_q), 2, d), 61), _rand((sum(lens_k), 1, d), 62), _rand((sum(lens_k), 1, d), 63)
+    dev = [t.to(cuda) for t in (q, k, v)]
+    out_dev = mindiesd.attention_forward_varlen(*dev, cu_q.to(cuda), cu_k.to(cuda), causal=causal).cpu()
+    out_host = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
+    assert torch.equal(out_dev, out_host)
+    _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
+
+
 def test_varlen_single_sequence_equals_dense(cuda):
     import mindiesd
     q, k, v = _rand((700, 2, 128), 14, mul=0.5), _rand((700, 2, 128), 15, mul=0.5), _rand((700, 2, 128), 16, mul=0.5)
