@@ -1016,8 +1016,6 @@ static int launch_fa(const FaParams& p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
-
-
 // cumulative lengths (device) -> the [B][4] table of the packed / general entry points, clamped to the tensors
 __global__ void varlen_meta_kernel(const int* cu_q, const int* cu_k, int B, int total_q, int total_k, int max_q,
                                    int max_k, int* meta) {
