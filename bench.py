@@ -229,6 +229,13 @@ def extra_causal_varlen(device, steps, warmup):
     cu = torch.tensor([0] + lens).cumsum(0).tolist()
     qt, kt, vt = (t[0].transpose(0, 1).contiguous() for t in (q, k, v))
     v_ms, _ = time_steps(lambda: mindiesd.attention_forward_varlen(qt, kt, vt, cu, cu), steps, warmup)
+    # many short sequences, cumulative lengths as host lists and as device tensors (no host read-back of the lengths)
+    nseq, slen = 63, 512
+    cu_s = [i * slen for i in range(nseq + 1)]
+    cu_d = torch.tensor(cu_s, dtype=torch.int32, device=device)
+    qp, kp, vp = (t[:nseq * slen] for t in (qt, kt, vt))
+    h_ms, _ = time_steps(lambda: mindiesd.attention_forward_varlen(qp, kp, vp, cu_s, cu_s), steps, warmup)
+    d_ms, _ = time_steps(lambda: mindiesd.attention_forward_varlen(qp, kp, vp, cu_d, cu_d), steps, warmup)
     # boolean masks, all true (timing of the mask path itself): one row shared by all queries, and a full [S, S] one
     pad = torch.ones(1, 1, 1, s, dtype=torch.bool, device=device).expand(1, 1, s, s)
     p_ms, _ = time_steps(lambda: flash_attention(q, k, v, d ** -0.5, "BNSD", attn_mask=pad), steps, warmup)
@@ -241,6 +248,7 @@ def extra_causal_varlen(device, steps, warmup):
     return {"workload": "bf16 B1 N12 S32760 D128: causal; and packed as 7 sequences " + str(lens),
             "causal_ms": cm, "causal_tflops_unmasked_work": causal_flops / cm / 1e9,
             "varlen_ms": vm, "varlen_tflops": varlen_flops / vm / 1e9,
+            "packed_63x512_host_lists_ms": median(h_ms), "packed_63x512_device_cu_seqlens_ms": median(d_ms),
             "key_padding_mask_ms": median(p_ms), "full_mask_ms": median(f_ms),
             "full_mask_tflops": attn_flops(cfg) / median(f_ms) / 1e9}
 

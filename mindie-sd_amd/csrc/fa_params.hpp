@@ -64,8 +64,10 @@ __device__ __forceinline__ bool packed_find_tile(const int* seq_meta, int nseq, 
       const int first = base + incl - t;
       const unsigned long long hit = __ballot(t > 0 && i >= first && i < first + t);
       const int l = __ffsll((long long)hit) - 1;  // exactly one lane holds tile i
-      seq = c0 + l;
-      tile = i - __shfl(first, l, 64);
+      // (handed back in scalar registers: everything the caller derives from them - pointers, sequence lengths, loop
+      // bounds - stays wave-uniform for the compiler as it is without the table)
+      seq = __builtin_amdgcn_readfirstlane(c0 + l);
+      tile = __builtin_amdgcn_readfirstlane(i - __shfl(first, l, 64));
       return true;
     }
     base += total;

@@ -97,7 +97,7 @@ __device__ __forceinline__ void tile_dma(__amdgpu_buffer_rsrc_t k_rsrc, __amdgpu
 // both passes is rounded to 16 bits once more than a one-pass walk would round it (a relative 2^-9 for bf16 on
 // the first pass's share of the row).
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false,
-          bool INIT = false>
+          bool INIT = false, bool PACKED = false>
 __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
@@ -114,7 +114,10 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   const int h = lane >> 5;
 
   // ---- which (batch, head, query tile): consecutive tiles of one head stay on one XCD -------
-  const bool packed = MODE && !SPARSE && p.packed_tiles > 0;
+  // PACKED (an instantiation of its own, so that the table lookup does not touch the code of the others): the grid
+  // holds p.packed_tiles query tiles per head, numbered through the sequences of p.seq_meta
+  static_assert(!PACKED || (MODE && !SPARSE && C::kBM == 128), "packed numbering: general dense mode, 128-row tiles");
+  constexpr bool packed = PACKED;
   const int q_tiles = packed ? p.packed_tiles : (p.Sq + C::kBM - 1) / C::kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
@@ -127,8 +130,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   int bn = work / q_tiles;
   int qt = work - bn * q_tiles;
   int b, n;
-  if (packed) {  // bn is the head; the tile's sequence comes from the table (kBM = 128 here)
-    static_assert(!MODE || SPARSE || C::kBM == 128, "packed numbering counts 128-row tiles");
+  if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
     n = bn;
     if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt)) return;
     if (p.causal) qt = (p.seq_meta[4 * b + 1] + C::kBM - 1) / C::kBM - 1 - qt;
@@ -1002,15 +1004,15 @@ static int launch_fa16(const FaParams& p, hipStream_t stream) {
 }
 
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE, int SCHED, int MODE = 0, bool GATHER = false,
-          bool INIT = false>
+          bool INIT = false, bool PACKED = false>
 static int launch_fa(const FaParams& p, hipStream_t stream) {
   using C = FaCfg<DT, NWAVES, QPW, BN, SPARSE>;
-  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE, GATHER, INIT>;
+  auto kern = fa_fwd_kernel<DT, NWAVES, QPW, BN, SPARSE, SCHED, MODE, GATHER, INIT, PACKED>;
   // per device and idempotent, so it is simply repeated on every launch
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes) != hipSuccess)
     return MSD_ERR_LAUNCH;
   const int q_tiles = (p.Sq + C::kBM - 1) / C::kBM;
-  const int total = (MODE && !SPARSE && p.packed_tiles > 0) ? p.N * p.packed_tiles : p.B * p.N * q_tiles;
+  const int total = PACKED ? p.N * p.packed_tiles : p.B * p.N * q_tiles;
   const int grid = ((total + 7) / 8) * 8;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kNT), C::kLdsBytes, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
@@ -1291,8 +1293,8 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
   if (tiles * N > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   p.packed_tiles = (int)tiles;
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
-  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
-  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
+  if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1, false, false, true>(p, stream);
+  return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1, false, false, true>(p, stream);
 }
 
 }  // extern "C"

@@ -40,7 +40,9 @@ struct HdCfg {
 
 constexpr float kTauHd = 8.0f;  // probabilities stay below 2^8: exact in fp32, representable in bf16 and fp16
 
-template <int DT, int DP>
+// PACKED (an instantiation of its own, so that the table lookup does not touch the code of the others): the grid holds
+// p.packed_tiles query tiles per head, numbered through the sequences of p.seq_meta.
+template <int DT, int DP, bool PACKED = false>
 __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const FaParams p, const int D) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using C = HdCfg<DP>;
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   const int h = lane >> 5;
 
   // consecutive query tiles of one head stay on one XCD (workgroups are dealt round-robin to the 8 XCDs)
-  const bool packed = p.packed_tiles > 0;  // the tiles of a head are numbered through the packed sequences
+  constexpr bool packed = PACKED;
   const int q_tiles = packed ? p.packed_tiles : (p.Sq + C::kBM - 1) / C::kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   const int bn = work / q_tiles;
   int qt = work - bn * q_tiles;
   int b, n;
-  if (packed) {
+  if constexpr (packed) {
     static_assert(C::kBM == 128, "packed numbering counts 128-row tiles");
     n = bn;
     if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt)) return;
@@ -327,17 +329,22 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int DP>
-static int launch_hd(const FaParams& p, int D, hipStream_t stream) {
+template <int DT, int DP, bool PACKED>
+static int launch_hd_p(const FaParams& p, int D, hipStream_t stream) {
   using C = HdCfg<DP>;
-  auto kern = fa_hd_kernel<DT, DP>;
+  auto kern = fa_hd_kernel<DT, DP, PACKED>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const long long total = p.packed_tiles > 0 ? (long long)p.N * p.packed_tiles
-                                             : (long long)p.B * p.N * ((p.Sq + C::kBM - 1) / C::kBM);
+  const long long total = PACKED ? (long long)p.N * p.packed_tiles
+                                 : (long long)p.B * p.N * ((p.Sq + C::kBM - 1) / C::kBM);
   if (total > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kern, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), C::kLds, stream, p, D);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
+}
+
+template <int DT, int DP>
+static int launch_hd(const FaParams& p, int D, hipStream_t stream) {
+  return p.packed_tiles > 0 ? launch_hd_p<DT, DP, true>(p, D, stream) : launch_hd_p<DT, DP, false>(p, D, stream);
 }
 
 int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream) {
