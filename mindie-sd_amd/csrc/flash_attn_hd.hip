@@ -40,9 +40,11 @@ struct HdCfg {
 
 constexpr float kTauHd = 8.0f;  // probabilities stay below 2^8: exact in fp32, representable in bf16 and fp16
 
-// PACKED (an instantiation of its own, so that the table lookup does not touch the code of the others): the grid holds
-// p.packed_tiles query tiles per head, numbered through the sequences of p.seq_meta.
-template <int DT, int DP, bool PACKED = false>
+// VAR selects what would otherwise be run-time branches around the tile loop (as such they cost the calls that do not
+// use them 2 % with the mask and 13 % with the table lookup): 0 = plain (causal and host-sized packed sequences are
+// run-time options), 1 = packed numbering - the grid holds p.packed_tiles query tiles per head, numbered through the
+// sequences of p.seq_meta -, 2 = boolean mask.
+template <int DT, int DP, int VAR = 0>
 __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const FaParams p, const int D) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using C = HdCfg<DP>;
@@ -59,7 +61,8 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   const int h = lane >> 5;
 
   // consecutive query tiles of one head stay on one XCD (workgroups are dealt round-robin to the 8 XCDs)
-  constexpr bool packed = PACKED;
+  constexpr bool packed = VAR == 1;
+  constexpr bool masked = VAR == 2;
   const int q_tiles = packed ? p.packed_tiles : (p.Sq + C::kBM - 1) / C::kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   int kv_lim = Skv;
   if (p.causal) kv_lim = max(0, min(Skv, q0 + C::kBM + causal_shift));
   const int tiles = (kv_lim + C::kBN - 1) / C::kBN;
-  const unsigned char* mask_g = p.mask ? p.mask + b * p.m_sb + n * p.m_sn : nullptr;
+  const unsigned char* mask_g = masked ? p.mask + b * p.m_sb + n * p.m_sn : nullptr;
 
   // V^T operand: the lane addresses key 4*h + (lane%16)/4 (+8 for the second read), head_dim 16*((lane/16)&1) +
   // 4*(lane%4) of a 32-wide block
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   };
 
   if (tiles > 0) {
-    if (mask_g && C::kBN <= Skv) mask_fetch(0);
+    if (masked && C::kBN <= Skv) mask_fetch(0);
     fetch(0);
     stash(0);
   }
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
   for (int t = 0; t < tiles; ++t) {
     const int stage = t & 1;
     const int key0 = t * C::kBN;
-    if (!mask_g && t + 1 < tiles) fetch(key0 + C::kBN);
+    if (!masked && t + 1 < tiles) fetch(key0 + C::kBN);
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
     MSD_LDS const char* vb_base = kb_base + C::kTileBytes;
 
@@ -205,20 +208,20 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
     const int qrow = q0 + wave * 32 + l32;
     const bool edge = key0 + C::kBN > Skv;
     const bool diag = p.causal && key0 + C::kBN - 1 > q0 + wave * 32 + causal_shift;
-    if (mask_g && !edge) {
+    if (masked && !edge) {
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (((mask_w[kb][r >> 2] >> (8 * (r & 3))) & 0xffu) == 0) sacc[kb][r] = -INFINITY;
     }
-    if (mask_g && t + 1 < tiles) {
+    if (masked && t + 1 < tiles) {
       if (key0 + 2 * C::kBN <= Skv) mask_fetch(key0 + C::kBN);
       fetch(key0 + C::kBN);
     }
     if (edge || diag) {
       const int last_visible = p.causal ? qrow + causal_shift : 0x7fffffff;
-      const unsigned char* mrow = (mask_g && edge) ? mask_g + (long long)min(qrow, Sq - 1) * p.m_sq : nullptr;
+      const unsigned char* mrow = (masked && edge) ? mask_g + (long long)min(qrow, Sq - 1) * p.m_sq : nullptr;
 #pragma unroll
       for (int kb = 0; kb < C::kNKB; ++kb)
 #pragma unroll
@@ -329,10 +332,11 @@ __global__ __launch_bounds__(256, (DP <= 128 ? 2 : 1)) void fa_hd_kernel(const F
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int DP, bool PACKED>
+template <int DT, int DP, int VAR>
 static int launch_hd_p(const FaParams& p, int D, hipStream_t stream) {
   using C = HdCfg<DP>;
-  auto kern = fa_hd_kernel<DT, DP, PACKED>;
+  constexpr bool PACKED = VAR == 1;
+  auto kern = fa_hd_kernel<DT, DP, VAR>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
   const long long total = PACKED ? (long long)p.N * p.packed_tiles
@@ -344,7 +348,8 @@ static int launch_hd_p(const FaParams& p, int D, hipStream_t stream) {
 
 template <int DT, int DP>
 static int launch_hd(const FaParams& p, int D, hipStream_t stream) {
-  return p.packed_tiles > 0 ? launch_hd_p<DT, DP, true>(p, D, stream) : launch_hd_p<DT, DP, false>(p, D, stream);
+  if (p.packed_tiles > 0) return launch_hd_p<DT, DP, 1>(p, D, stream);  // (never together with a mask)
+  return p.mask ? launch_hd_p<DT, DP, 2>(p, D, stream) : launch_hd_p<DT, DP, 0>(p, D, stream);
 }
 
 int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream) {
