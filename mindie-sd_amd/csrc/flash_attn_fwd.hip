@@ -318,7 +318,10 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   if (MODE && p.causal) kv_lim = max(0, min(Skv, q0 + C::kBM + causal_shift));
   const int dense_tiles = (kv_lim + BN - 1) / BN;
   const unsigned char* mask_g = nullptr;
-  if (MODE && p.mask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
+  // MODE 2 = general mode with a boolean mask: an instantiation of its own, because as a run-time test the mask words
+  // cost the causal and variable-length calls registers they do not use.
+  constexpr bool masked = MODE == 2;
+  if (masked) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
   // Boolean mask of a tile that lies wholly inside the sequence: the lane fetches the BN bytes of its own query row as
   // 16-byte words (any alignment: global loads take unaligned addresses) one tile ahead, into the set that belongs to
   // the tile's LDS stage, so they arrive with the tile's own data and cost no wait of their own.  The tile that runs
@@ -365,7 +368,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
     }
   } else {
     load_tile(0, 0);
-    if (MODE && mask_g && BN <= Skv) mask_fetch(0, std::integral_constant<int, 0>{});
+    if (masked && BN <= Skv) mask_fetch(0, std::integral_constant<int, 0>{});
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the LDS-DMA of this wave has landed
   __syncthreads();
@@ -380,7 +383,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
   auto tile_step = [&](auto stage_c, const int key0, const int next_key0, const bool active) {
     constexpr int stage = decltype(stage_c)::value;
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
-    if (MODE && !SPARSE && mask_g && next_key0 >= 0 && next_key0 + BN <= Skv)
+    if (masked && !SPARSE && next_key0 >= 0 && next_key0 + BN <= Skv)
       mask_fetch(next_key0, std::integral_constant<int, stage ^ 1>{});
     if (active) {
     MSD_LDS const char* kb_base = smem + stage * C::kStageBytes;
@@ -447,7 +450,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
         }
       }
       // boolean mask: one byte per (query, key); a lane tests the 16 x kNKB keys of its own query row
-      if (mask_g && !SPARSE && key0 + BN <= Skv) {
+      if (masked && !SPARSE && key0 + BN <= Skv) {
         // register r of block kb is key 32 kb + 8 (r / 4) + 4 h + r % 4: dword 2 (r / 4) + h of the block's 32 bytes
 #pragma unroll
         for (int qb = 0; qb < C::kNQB; ++qb)
@@ -461,7 +464,7 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
               for (int j = 0; j < 4; ++j)
                 if (((w >> (8 * j)) & 0xffu) == 0) sacc[kb][qb][4 * g4 + j] = -INFINITY;
             }
-      } else if (mask_g) {
+      } else if (masked) {
 #pragma unroll
         for (int qb = 0; qb < C::kNQB; ++qb) {
           const int qrow = min(q0 + wave * QPW + qb * 32 + l32, Sq - 1);
@@ -1255,6 +1258,10 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
+  if (mask) {
+    if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 2>(p, stream);
+    return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 2>(p, stream);
+  }
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
 }
