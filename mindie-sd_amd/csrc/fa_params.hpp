@@ -45,21 +45,22 @@ struct FaParams {
 
 #if defined(__HIP_DEVICE_COMPILE__)
 // Packed numbering of the query tiles (FaParams::packed_tiles): which sequence tile i of a head belongs to and which
-// of that sequence's 128-row tiles it is.  Every lane of the wave takes one sequence of a group of 64, the running
+// of that sequence's tiles of `rows` query rows it is.  Every lane of the wave takes one sequence of a group of 64, the running
 // sum of the tile counts is a wave scan; the result is wave-uniform.  False: i lies past the last tile.
-__device__ __forceinline__ bool packed_find_tile(const int* seq_meta, int nseq, int i, int& seq, int& tile) {
+__device__ __forceinline__ bool packed_find_tile(const int* seq_meta, int nseq, int i, int& seq, int& tile,
+                                                 int rows = 128) {
   const int lane = threadIdx.x & 63;
   int base = 0;
   for (int c0 = 0; c0 < nseq; c0 += 64) {
     const int s = c0 + lane;
-    const int t = s < nseq ? (seq_meta[4 * s + 1] + 127) / 128 : 0;
+    const int t = s < nseq ? (seq_meta[4 * s + 1] + rows - 1) / rows : 0;
     int incl = t;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const int u = __shfl_up(incl, d, 64);
       if (lane >= d) incl += u;
     }
-    const int total = __shfl(incl, 63, 64);
+    const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63, 64));  // (scalar: the branch below is uniform)
     if (i < base + total) {
       const int first = base + incl - t;
       const unsigned long long hit = __ballot(t > 0 && i >= first && i < first + t);

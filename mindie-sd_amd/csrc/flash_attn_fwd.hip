@@ -6,9 +6,10 @@
 // rainfusionattention (csrc/plugin/block_sparse_attention.cpp:31-121,
 // csrc/plugin/rainfusionattention.cpp:27-64).
 //
-// Two kernels share the algorithm: fa_fwd16_kernel (plain dense attention, 16x16x32 matrix instruction) and
-// fa_fwd_kernel (block-sparse, masked, causal and packed variable-length attention and the tuning variants of the
-// dense case, 32x32x16 instruction).  What follows describes fa_fwd_kernel; fa_fwd16_kernel states its differences.
+// Two kernels share the algorithm: fa_fwd16_kernel (16x16x32 matrix instruction: plain dense attention, and causal
+// and packed variable-length attention without a boolean mask from 1024 query rows on) and fa_fwd_kernel (32x32x16
+// instruction: block-sparse and masked attention, the short causal / variable-length cases and the tuning variants
+// of the dense case).  What follows describes fa_fwd_kernel; fa_fwd16_kernel states its differences.
 //
 // Algorithm: single pass, online softmax.  One workgroup owns BM = NWAVES*QPW query rows of one
 // (batch, head); it walks the key/value sequence in tiles of BN keys staged in LDS (double
@@ -683,7 +684,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 // those waves compute on zeros and store nothing); the key tiles are the 128-key blocks of the pair's list
 // (p.blk_idx / p.blk_cnt indexed by pair) instead of the whole sequence.  Besides the normalised rows it writes
 // p.state, the log2-domain log-sum-exp the second pass resumes from.  GATHER as in fa_fwd_kernel.
-template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false>
+//
+// GEN 1: the general mode without a boolean mask: per-sequence lengths and token offsets from p.seq_meta and / or a
+// causal mask aligned to the bottom-right corner.  No per-row flags are needed for it: a row either sees key 0, which
+// lies in its first tile, or (causal with more queries than keys) no key at all, and the first tile's rule for the
+// reference maximum covers both.  GEN 2: the same with the packed tile numbering of p.packed_tiles (256-row tiles).
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0>
 __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
@@ -701,17 +707,39 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int g = lane >> 4;
 
   static_assert(!PAIR || NWAVES == 8, "a pair is two groups of four waves");
-  const int q_tiles = PAIR ? p.NP : (p.Sq + kBM - 1) / kBM;
-  const int total = p.B * p.N * q_tiles;
+  constexpr bool gen = GEN != 0, packed = GEN == 2;
+  static_assert(!gen || (!PAIR && !GATHER), "general mode: dense tensors in their own order");
+  const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
+  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   const int per_xcd = (total + 7) / 8;
   const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
-  const int bn = work / q_tiles;
-  const int qt = work - bn * q_tiles;
-  const int b = bn / p.N;
-  const int n = bn - b * p.N;
+  int bn = work / q_tiles;
+  int qt = work - bn * q_tiles;
+  int b, n;
+  if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
+    n = bn;
+    if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt, kBM)) return;
+    if (p.causal) qt = (p.seq_meta[4 * b + 1] + kBM - 1) / kBM - 1 - qt;
+    bn = b * p.N + n;
+  } else {
+    if (gen && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
+    b = bn / p.N;
+    n = bn - b * p.N;
+  }
   const int nkv = n / (p.N / p.Nkv);
-  const int Sq = p.Sq, Skv = p.Skv;
+  int Sq = p.Sq, Skv = p.Skv;
+  long long q_tok0 = 0, k_tok0 = 0;  // general mode: first token of the sequence in packed tensors
+  if constexpr (gen) {
+    if (p.seq_meta) {
+      const int* meta = p.seq_meta + 4 * b;
+      Sq = meta[1];
+      Skv = meta[3];
+      if (qt * kBM >= Sq) return;  // the grid is sized for the longest sequence
+      q_tok0 = meta[0];
+      k_tok0 = meta[2];
+    }
+  }
   // first query row of this wave; rows at or beyond row_end do not exist (tail of the sequence / of the block)
   int row0 = qt * kBM + wave * 32, row_end = Sq;
   if constexpr (PAIR) {
@@ -721,10 +749,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     if (qblk < 0) row0 = 0;
   }
 
-  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
-  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
-  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
-  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn + q_tok0 * p.q_ss;
+  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn + k_tok0 * p.k_ss;
+  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn + k_tok0 * p.v_ss;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn + q_tok0 * p.o_ss;
 
   // ---- Q^T operand, resident: lane (c, g) holds query 16*nq + c, head_dim 32*ks + 8*g .. +8 --------------
   X8 qf[2][4];
@@ -763,10 +791,11 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   }
 
   // ---- global -> LDS staging (LDS-DMA; swizzles applied on the global side) -------------------------------
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kg, 0, (int)(((long long)(Skv - 1) * p.k_ss + 128) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vg, 0, (int)(((long long)(Skv - 1) * p.v_ss + 128) * 2), 0x00020000);
+  // (a sequence without keys exposes nothing: every row reads as zeros and no tile is computed)
+  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + 128) * 2);
+  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + 128) * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, k_range, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, v_range, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
   int k_voff, v_voff;
   {
@@ -793,7 +822,11 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     v_lds[db] = (unsigned)(uintptr_t)smem + 2 * kTileBytes + (4 * g + (c >> 2)) * kRowBytes +
                 ((db ^ (4 * (g & 1) + (c >> 2))) << 5) + 8 * (c & 3);
 
-  const int tiles = (Skv + BN - 1) / BN;
+  // causal: query i sees keys <= i + causal_shift; the last row of this workgroup bounds the tiles it walks
+  const int causal_shift = Skv - Sq;
+  const bool causal = gen && p.causal;
+  const int kv_lim = causal ? max(0, min(Skv, qt * kBM + kBM + causal_shift)) : Skv;
+  const int tiles = (kv_lim + BN - 1) / BN;
   // PAIR: the ids of the list are fetched with scalar loads two tiles ahead of their use
   int l_n = 0, id_a = -1, id_b = -1;  // id_a: the tile being computed (already requested), id_b: the one after it
   const int* l_ptr = nullptr;
@@ -858,6 +891,20 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
             sacc[kb][0][i] = -INFINITY;
             sacc[kb][1][i] = -INFINITY;
           }
+    }
+
+    // ---- causal: keys beyond the diagonal (the tiles that cross it for some row of this wave) ------------------
+    if constexpr (gen) {
+      if (causal && key0 + BN - 1 > row0 + causal_shift) {
+        const int lim = row0 + c + causal_shift - key0 - 4 * g;  // visible: 16 * kb + i <= lim (+16 for nq = 1)
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (16 * kb + i > lim) sacc[kb][0][i] = -INFINITY;
+            if (16 * kb + i > lim + 16) sacc[kb][1][i] = -INFINITY;
+          }
+      }
     }
 
     // ---- online softmax (exp2 domain, lazily moved reference maximum; see fa_fwd_kernel) ---------------------
@@ -995,13 +1042,14 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false>
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0>
 static int launch_fa16(const FaParams& p, hipStream_t stream) {
   constexpr int kLds = 4 * 128 * 256;  // two K and two V stages of 128 keys
-  auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER>;
+  auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER, GEN>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const int total = p.B * p.N * (PAIR ? p.NP : (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
+  const int total = GEN == 2 ? p.N * p.packed_tiles
+                             : p.B * p.N * (PAIR ? p.NP : (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
   hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
@@ -1039,6 +1087,8 @@ using namespace msd;
 extern "C" {
 
 constexpr int kShortKv = 384;  // dense calls with at most this many keys run on the 4-wave kernel (see below)
+// general mode: query rows (of the longest sequence; packed: of the average one) from which the 8-wave kernel is used
+constexpr int kGen16MinRows = 1024;
 
 static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
                         int Nkv, int Sq, int Skv, int D, const long long* st, float scale, bool any_head_dim = false) {
@@ -1262,6 +1312,12 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
     if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 2>(p, stream);
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 2>(p, stream);
   }
+  // Without a mask, long sequences run on the 16x16x32 kernel's general instantiation (256-row tiles); short ones
+  // fill the chip better with the 128-row tiles of the 4-wave kernel.
+  if (Sq >= kGen16MinRows && Skv > kShortKv) {
+    if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 1>(p, stream);
+    return launch_fa16<MSD_DTYPE_F16, 8, false, false, 1>(p, stream);
+  }
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
 }
@@ -1300,6 +1356,12 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
   if (tiles * N > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   p.packed_tiles = (int)tiles;
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
+  // long sequences on average: the 8-wave kernel, whose tiles are 256 rows
+  if (total_q / B >= kGen16MinRows && total_k / B > kShortKv) {
+    p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
+    if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 2>(p, stream);
+    return launch_fa16<MSD_DTYPE_F16, 8, false, false, 2>(p, stream);
+  }
   if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1, false, false, true>(p, stream);
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1, false, false, true>(p, stream);
 }

@@ -73,7 +73,9 @@ def test_mask_dtypes_and_fully_masked_rows(cuda):
     assert torch.equal(out[:, :, rows], v[:, :, 17:18].expand(1, 2, 129, 128))  # one visible key: the output is its value row
 
 
-@pytest.mark.parametrize("sq,skv", [(256, 256), (300, 300), (77, 500), (500, 77), (1000, 1300)])
+# (from 1024 query rows on, calls without a mask run on the 8-wave kernel's general instantiation)
+@pytest.mark.parametrize("sq,skv", [(256, 256), (300, 300), (77, 500), (500, 77), (1000, 1300), (1100, 1100),
+                                    (1300, 1800), (1800, 1300), (1025, 2047), (1536, 385)])
 def test_causal_bottom_right(cuda, sq, skv):
     from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
     q, k, v = _rand((1, 4, sq, 128), 8), _rand((1, 2, skv, 128), 9), _rand((1, 2, skv, 128), 10)
@@ -146,6 +148,38 @@ def test_varlen_many_sequences_device_table(cuda, d, causal):
     out_host = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
     assert torch.equal(out_dev, out_host)
     _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_varlen_long_sequences(cuda, causal, dtype):
+    """Sequences of 1024 query tokens and more take the 8-wave kernel (256-row tiles): lengths around the tile edges,
+    key counts above and below the query counts (causal rows without any visible key give zeros), a sequence without
+    keys and one without queries, grouped heads.  Host lists size the grid by the longest sequence; device tables
+    of long sequences number the tiles through the table."""
+    import mindiesd
+    lens_q, lens_k = [1500, 1, 0, 1100, 300, 40, 1281], [1500, 700, 5, 1300, 2000, 0, 1000]
+    cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+    cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+    q, k, v = (_rand((sum(lens_q), 4, 128), 31, dtype), _rand((sum(lens_k), 2, 128), 32, dtype),
+               _rand((sum(lens_k), 2, 128), 33, dtype))
+    ref = attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal)
+    dev = [t.to(cuda) for t in (q, k, v)]
+    out = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
+    _check(out, ref)
+    o5 = int(cu_q[5])
+    assert not out[o5:o5 + 40].any()          # the sequence without keys
+    # device tables: 4 long sequences (average >= 1024 tokens), tiles numbered through the table
+    lq2, lk2 = [1500, 1100, 1281, 2049], [1500, 1300, 1000, 2049]
+    cq2 = torch.tensor([0] + lq2).cumsum(0).to(torch.int32)
+    ck2 = torch.tensor([0] + lk2).cumsum(0).to(torch.int32)
+    q2, k2, v2 = (_rand((sum(lq2), 4, 128), 34, dtype), _rand((sum(lk2), 2, 128), 35, dtype),
+                  _rand((sum(lk2), 2, 128), 36, dtype))
+    dev2 = [t.to(cuda) for t in (q2, k2, v2)]
+    out_dev = mindiesd.attention_forward_varlen(*dev2, cq2.to(cuda), ck2.to(cuda), causal=causal).cpu()
+    out_host = mindiesd.attention_forward_varlen(*dev2, cq2.tolist(), ck2.tolist(), causal=causal).cpu()
+    assert torch.equal(out_dev, out_host)
+    _check(out_dev, attention_varlen(q2, k2, v2, cq2.tolist(), ck2.tolist(), causal=causal))
 
 
 def test_varlen_single_sequence_equals_dense(cuda):
