@@ -123,6 +123,22 @@ def test_fp8_attention_vs_oracle(cuda, layout, s, recipe, p_rule):
 
 
 @pytest.mark.parametrize("recipe", ["pow2", "amax"])
+@pytest.mark.parametrize("sq,skv", [(700, 1100), (1300, 300), (130, 2049)])
+def test_fp8_attention_unequal_query_and_key_lengths(cuda, sq, skv, recipe):
+    """Cross attention: the query and key / value sequences have lengths of their own."""
+    from mindiesd.layers.quant import fp8_attention_forward
+    q, _, _ = _outlier_inputs((1, 2, sq, 128), seed=sq)
+    _, k, v = _outlier_inputs((1, 2, skv, 128), seed=skv)
+    want = oq.fp8_attention(q, k, v, pow2=recipe == "pow2")
+    out = fp8_attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), layout="BNSD", recipe=recipe).cpu()
+    assert out.shape == q.shape
+    assert cosine(out, want) >= 0.999
+    mirror = oq.fp8_attention(q, k, v, pow2=recipe == "pow2", requant_p=True, p_rule="linear")
+    assert cosine(out, mirror) >= 0.99999
+    assert (out.float() - mirror.float()).abs().max() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
+
+
+@pytest.mark.parametrize("recipe", ["pow2", "amax"])
 @pytest.mark.parametrize("s", [1100, 640])
 def test_fp8_attention_k_scale_per_256_tokens(cuda, s, recipe):
     """K quantised per 256-token block (the K recipe of the reference's FP8RotateQuantFA, layer.py:297-302): scales from
