@@ -459,8 +459,7 @@ int mindiesd_mxfp8_gemm(const void* a, const void* a_scale, const void* w, const
   p.M = M; p.K = K; p.Nw = Nw; p.Nout = swiglu ? Nw / 2 : Nw;
   p.tiles_m = (M + 255) / 256;
   p.tiles_n = swiglu ? (Nw / 2 + 127) / 128 : (Nw + 255) / 256;
-  constexpr int kLds = 8 * 16384 + 2 * 8192 + 1024;  // ring of eight 16 KiB units + two scale chunk buffers + scrap;
-                                                             // the output staging (4 x 32 rows x 264 B) reuses the ring
+  constexpr int kLds = 8 * 16384 + 2 * 8192 + 1024;  // ring of eight 16 KiB units + two scale chunk buffers + scrap
   const int total = p.tiles_m * p.tiles_n;
   const int grid = (total + 7) / 8 * 8;
 #define MSD_LAUNCH_GEMM(DTV, SW)                                                                                   \
