@@ -178,12 +178,12 @@ def extra_dense_1p3b(device, steps, warmup):
 
 
 def extra_head_dims(device, steps, warmup):
-    """Dense attention at head dims other than 128 at a 17776-token sequence: 64 (its own kernel) and 256 (the general
-    kernel)."""
+    """Dense attention at head dims other than 128 at a 17776-token sequence: 64 (its own kernel), 72 and 96 (computed
+    as head_dim 128 on the dense kernel) and 256 (the general kernel)."""
     import torch
     import mindiesd
-    res = {"workload": "dense bf16 B1 S17776 (13x30x45 latent tokens + 226 text tokens), N48 D64 / N12 D256"}
-    for n, d in ((48, 64), (12, 256)):
+    res = {"workload": "dense bf16 B1 S17776 (13x30x45 latent tokens + 226 text tokens), N48 D64 / N48 D72 / N32 D96 / N12 D256"}
+    for n, d in ((48, 64), (48, 72), (32, 96), (12, 256)):
         g = torch.Generator(device=device).manual_seed(7)
         q, k, v = ((torch.randn((1, n, 17776, d), device=device, generator=g) * 0.5).to(torch.bfloat16) for _ in range(3))
         ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), steps, warmup)

@@ -41,6 +41,7 @@ struct FaParams {
   int causal;                 // key j is visible to query i iff j <= i + (Skv - Sq) (mask aligned bottom-right)
   const unsigned char* mask;  // optional boolean mask, non-zero = attend; keys contiguous
   long long m_sb, m_sn, m_sq; // its element strides over batch, head (0 = broadcast) and query
+  int head_dim;               // DPAD instantiations of fa_fwd16_kernel: the tensors' head_dim (a multiple of 8 below 128)
 };
 
 #if defined(__HIP_DEVICE_COMPILE__)

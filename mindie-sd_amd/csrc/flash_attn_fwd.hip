@@ -689,7 +689,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 // causal mask aligned to the bottom-right corner.  No per-row flags are needed for it: a row either sees key 0, which
 // lies in its first tile, or (causal with more queries than keys) no key at all, and the first tile's rule for the
 // reference maximum covers both.  GEN 2: the same with the packed tile numbering of p.packed_tiles (256-row tiles).
-template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0>
+//
+// DPAD: tensors whose head_dim lies between 64 and 128 (p.head_dim, a multiple of 8), computed as head_dim 128: the
+// query operand is zero from p.head_dim on, and the lanes that would stage the 16-byte chunks of K and V past it
+// request an offset beyond the buffers' range instead, for which the DMA writes zeros without touching memory.  The
+// output columns past p.head_dim are not stored.
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0, bool DPAD = false>
 __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using E = Elem<DT>;
@@ -764,8 +769,14 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     const T* src = qg + (long long)qsrc * p.q_ss + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      X8 v = *(const X8*)(src + 32 * ks);
-      if (!ok) v = X8{0};
+      X8 v;
+      if constexpr (DPAD) {
+        const bool in = ok && 32 * ks + 8 * g < p.head_dim;  // (a chunk of 8 lies wholly inside or outside)
+        v = in ? *(const X8*)(src + 32 * ks) : X8{0};
+      } else {
+        v = *(const X8*)(src + 32 * ks);
+        if (!ok) v = X8{0};
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = E::from_float((float)v[j] * p.scale_log2);
       qf[nq][ks] = v;
@@ -792,8 +803,9 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
 
   // ---- global -> LDS staging (LDS-DMA; swizzles applied on the global side) -------------------------------
   // (a sequence without keys exposes nothing: every row reads as zeros and no tile is computed)
-  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + 128) * 2);
-  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + 128) * 2);
+  const int row_elems = DPAD ? p.head_dim : 128;
+  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + row_elems) * 2);
+  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + row_elems) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, k_range, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, v_range, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
@@ -801,8 +813,13 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   {
     const int row = 4 * wave + (lane >> 4);  // groups of one wave lie 4 * NWAVES rows apart: same swizzles
     const int pc = lane & 15;                // physical 16-byte chunk this lane fills
-    k_voff = row * k_row_bytes + ((pc ^ (row & 15)) << 4);
-    v_voff = row * v_row_bytes + (((((pc >> 1) ^ (row & 7)) << 1) | (pc & 1)) << 4);
+    const int kc = pc ^ (row & 15), vc = (((pc >> 1) ^ (row & 7)) << 1) | (pc & 1);  // logical chunks of the row
+    k_voff = row * k_row_bytes + (kc << 4);
+    v_voff = row * v_row_bytes + (vc << 4);
+    if constexpr (DPAD) {  // chunks past the head_dim: an offset beyond every range, the DMA writes zeros for them
+      if (kc * 8 >= p.head_dim) k_voff = 0x7ffffff0;
+      if (vc * 8 >= p.head_dim) v_voff = 0x7ffffff0;
+    }
   }
   auto load_tile = [&](int key0, int stage) {
     tile_dma<BN / 4 / NWAVES, NWAVES>(k_rsrc, v_rsrc, smem + stage * kTileBytes, smem + (2 + stage) * kTileBytes, k_voff,
@@ -1033,7 +1050,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     const int qrow = row0 + row;
     const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16);
     const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c16 * 16 + 8);
-    if (qrow < row_end) {
+    if (qrow < row_end && (!DPAD || c16 * 8 < p.head_dim)) {
       i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
       const int orow = GATHER ? p.tok[qrow] : qrow;
       *(i32x4_t*)(og + (long long)orow * p.o_ss + c16 * 8) = v;
@@ -1042,10 +1059,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0>
+template <int DT, int NWAVES = 8, bool PAIR = false, bool GATHER = false, int GEN = 0, bool DPAD = false>
 static int launch_fa16(const FaParams& p, hipStream_t stream) {
   constexpr int kLds = 4 * 128 * 256;  // two K and two V stages of 128 keys
-  auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER, GEN>;
+  auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER, GEN, DPAD>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
   const int total = GEN == 2 ? p.N * p.packed_tiles
@@ -1226,6 +1243,15 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   if (rc != MSD_OK) return rc;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream);
+  // Head dims between 64 and 128 run as head_dim 128 on the 16x16x32 kernel (the part of the matrix work spent on
+  // the padding costs less than the general kernel's staging through registers: 72 -> 580 vs 730 TFLOP/s of real
+  // work, 112 -> 800 vs 1130), when the 256-byte rows the DMA fetches stay inside the kernel's 32-bit offsets.
+  if (D > 64 && D < 128 && Skv > kShortKv && (long long)Skv * k_ss * 2 < 0x7fffff00ll &&
+      (long long)Skv * v_ss * 2 < 0x7fffff00ll) {  // (below the offset that stands for "no data" in the kernel)
+    p.head_dim = D;
+    if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 0, true>(p, stream);
+    return launch_fa16<MSD_DTYPE_F16, 8, false, false, 0, true>(p, stream);
+  }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   // A few key tiles per query tile (cross attention over a short text): the launch is mostly reading Q and writing O,
   // and two 4-wave workgroups per CU overlap one's memory phases with the other's tiles better than one 8-wave

@@ -132,6 +132,36 @@ def test_head_dim_64_dense_kernel_against_general_kernel_and_oracle(cuda, sq, sk
     _check(out[:, rows].cpu(), ref, max_abs=tol, min_cos=0.9999 if dtype == torch.bfloat16 else 0.99999)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [72, 88, 96, 120])
+@pytest.mark.parametrize("sq,skv", [(2311, 3001), (33, 4100), (600, 385)])
+def test_head_dims_between_64_and_128_on_the_dense_kernel(cuda, d, sq, skv, dtype):
+    """Dense attention without a mask at these head dims runs as head_dim 128 on the 16x16x32 kernel; an all-true mask
+    sends the same inputs through the general kernel.  q, k, v are views of 128-wide buffers whose columns past the
+    head_dim hold NaN: nothing beyond a row's own elements may reach the result.  Grouped-query heads, BSND storage."""
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    def in_nan_buffer(t):
+        buf = torch.full(t.shape[:-1] + (128,), float("nan"), dtype=t.dtype, device=cuda)
+        buf[..., :d] = t.to(cuda)
+        return buf[..., :d]
+    q, k, v = _rand((1, sq, 6, d), 70, dtype), _rand((1, skv, 2, d), 71, dtype), _rand((1, skv, 2, d), 72, dtype)
+    dq, dk, dv = in_nan_buffer(q), in_nan_buffer(k), in_nan_buffer(v)
+    out, lse = flash_attention(dq, dk, dv, d ** -0.5, "BSND", return_lse=True)
+    assert not torch.isnan(out.float()).any()
+    gen, lse_g = flash_attention(dq, dk, dv, d ** -0.5, "BSND", return_lse=True,
+                                 attn_mask=torch.ones(sq, skv, dtype=torch.bool, device=cuda))
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3
+    assert (out.float() - gen.float()).abs().max().item() <= tol
+    assert (lse - lse_g).abs().max().item() < 1e-3
+    rows = sorted({0, 1, 15, 16, 31, 32, sq // 2, sq - 2, sq - 1} & set(range(sq)))
+    kk, vv = k.repeat_interleave(3, dim=2), v.repeat_interleave(3, dim=2)
+    ref = attention_math(q[:, rows], kk, vv, None, d ** -0.5, head_first=False)
+    _check(out[:, rows].cpu(), ref, max_abs=tol, min_cos=0.9999 if dtype == torch.bfloat16 else 0.99999)
+    # contiguous tensors (rows d elements apart: the 256-byte fetch of a row overlaps the next rows) give the same
+    out_c = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BSND")
+    assert torch.equal(out_c, out)
+
+
 def test_rejected_head_dims(cuda):
     import mindiesd
     from mindiesd.utils.exception import ParametersInvalid
