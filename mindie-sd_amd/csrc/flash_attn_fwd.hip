@@ -689,6 +689,12 @@ __global__ __launch_bounds__(NWAVES * 64, (QPW == 32 ? 2 : 1)) void fa_fwd_kerne
 // causal mask aligned to the bottom-right corner.  No per-row flags are needed for it: a row either sees key 0, which
 // lies in its first tile, or (causal with more queries than keys) no key at all, and the first tile's rule for the
 // reference maximum covers both.  GEN 2: the same with the packed tile numbering of p.packed_tiles (256-row tiles).
+// GEN 3: a boolean mask over the keys that all queries of a (batch, head) share (p.mask with m_sq = 0, a key-padding
+// mask; neither causal nor per-sequence lengths).  The 128 bytes of the next tile are fetched during the second product and reduced to four
+// 32-bit words of visible keys in scalar registers; a tile with all of its keys visible runs the plain code, the
+// others test their scores against the words.  The rule of the first tile stays in force until a tile has shown the
+// wave a key: that tile holds the first visible key, which every row sees, so once more no row needs a state of
+// its own.
 //
 // DPAD: tensors whose head_dim lies between 64 and 128 (p.head_dim, a multiple of 8), computed as head_dim 128: the
 // query operand is zero from p.head_dim on, and the lanes that would stage the 16-byte chunks of K and V past it
@@ -712,7 +718,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int g = lane >> 4;
 
   static_assert(!PAIR || NWAVES == 8, "a pair is two groups of four waves");
-  constexpr bool gen = GEN != 0, packed = GEN == 2;
+  constexpr bool gen = GEN != 0, packed = GEN == 2, keymask = GEN == 3;
   static_assert(!gen || (!PAIR && !GATHER), "general mode: dense tensors in their own order");
   const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
@@ -728,14 +734,14 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     if (p.causal) qt = (p.seq_meta[4 * b + 1] + kBM - 1) / kBM - 1 - qt;
     bn = b * p.N + n;
   } else {
-    if (gen && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
+    if (gen && !keymask && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
     b = bn / p.N;
     n = bn - b * p.N;
   }
   const int nkv = n / (p.N / p.Nkv);
   int Sq = p.Sq, Skv = p.Skv;
   long long q_tok0 = 0, k_tok0 = 0;  // general mode: first token of the sequence in packed tensors
-  if constexpr (gen) {
+  if constexpr (gen && !keymask) {
     if (p.seq_meta) {
       const int* meta = p.seq_meta + 4 * b;
       Sq = meta[1];
@@ -841,7 +847,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
 
   // causal: query i sees keys <= i + causal_shift; the last row of this workgroup bounds the tiles it walks
   const int causal_shift = Skv - Sq;
-  const bool causal = gen && p.causal;
+  const bool causal = gen && !keymask && p.causal;  // (with a key mask: neither causal nor per-sequence lengths)
   const int kv_lim = causal ? max(0, min(Skv, qt * kBM + kBM + causal_shift)) : Skv;
   const int tiles = (kv_lim + BN - 1) / BN;
   // PAIR: the ids of the list are fetched with scalar loads two tiles ahead of their use
@@ -861,9 +867,42 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   __syncthreads();
   bool first = true;
 
+  // ---- key mask (GEN 3): words of visible keys of the current tile; bit l of word j = key 4 * l + j ------------
+  unsigned kvis[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  unsigned kraw = 0;  // the lane's four mask bytes of the tile that comes next (lanes 0 .. 31)
+  const unsigned char* mask_g = nullptr;
+  if constexpr (keymask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
+  auto mask_request = [&](int key0) __attribute__((always_inline)) {  // the load only
+    if constexpr (keymask) {
+      kraw = 0;
+      const int k4 = key0 + 4 * (lane & 31);
+      if (key0 + BN <= Skv) {
+        __builtin_memcpy(&kraw, mask_g + k4, 4);  // (any alignment)
+      } else {                                    // the tile that runs past the row: byte by byte, inside the row
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned byte = mask_g[min(k4 + j, Skv - 1)];
+          kraw |= (k4 + j < Skv ? byte : 0u) << (8 * j);
+        }
+      }
+    }
+  };
+  auto mask_reduce = [&]() __attribute__((always_inline)) {  // bytes -> words in scalar registers
+    if constexpr (keymask) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        kvis[j] = (unsigned)__builtin_amdgcn_ballot_w64(lane < 32 && ((kraw >> (8 * j)) & 0xffu) != 0);
+    }
+  };
+  if constexpr (keymask) {
+    if (tiles > 0) mask_request(0);
+    mask_reduce();
+  }
+
   auto tile_step = [&](auto stage_c, const int key0, const int next_key0) {
     constexpr int stage = decltype(stage_c)::value;
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+    const unsigned kv_all = kvis[0] & kvis[1] & kvis[2] & kvis[3];
 
     // ---- S^T = K Q^T: 16 accumulation chains; operand reads in groups of 2 key blocks of one 32-wide head_dim
     // step, kAhead groups ahead of the matrix instructions that use them (ring of kAhead + 1) -----------------
@@ -924,8 +963,25 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
       }
     }
 
+    // ---- key mask: tiles that hide some of their keys ----------------------------------------------------------
+    if constexpr (keymask) {
+      if (kv_all != 0xffffffffu) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned w = kvis[i] >> g;  // key 16 * kb + 4 * g + i is bit 4 * kb + g of word i
+#pragma unroll
+          for (int kb = 0; kb < 8; ++kb)
+            if (!((w >> (4 * kb)) & 1u)) {
+              sacc[kb][0][i] = -INFINITY;
+              sacc[kb][1][i] = -INFINITY;
+            }
+        }
+      }
+    }
+
     // ---- online softmax (exp2 domain, lazily moved reference maximum; see fa_fwd_kernel) ---------------------
     X8 pf[2][4];
+    bool seen = !keymask;  // key mask: this tile showed some row of the wave a key (all rows share the mask)
 #pragma unroll
     for (int nq = 0; nq < 2; ++nq) {
       float mx = sacc[0][nq][0];
@@ -933,6 +989,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
       for (int kb = 0; kb < 8; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
+      if constexpr (keymask) seen = seen || __builtin_amdgcn_ballot_w64(mx > -INFINITY) != 0;
       // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
       float delta = 0.f, alpha = 1.f;
       int moved = 0;
@@ -975,6 +1032,9 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
         dst[2 * d4 + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(a);
       }
     };
+    if constexpr (keymask) {
+      if (next_key0 >= 0) mask_request(next_key0);  // lands during the second product
+    }
     issue(std::integral_constant<int, 0>{}, vf[0]);
     static_for<8>([&](auto step_c) __attribute__((always_inline)) {
       constexpr int s = decltype(step_c)::value;
@@ -1000,8 +1060,9 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
       }
     });
 
-    first = false;
+    first = first && !seen;  // (without a key mask: false from the first tile on)
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next tile has landed
+    mask_reduce();
     __syncthreads();
   };
   if constexpr (PAIR) {
@@ -1334,6 +1395,10 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
+  if (mask && m_sq == 0 && !causal && !seq_meta && Sq >= kGen16MinRows && Skv > kShortKv) {  // one mask row for all queries: the 8-wave kernel
+    if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 3>(p, stream);
+    return launch_fa16<MSD_DTYPE_F16, 8, false, false, 3>(p, stream);
+  }
   if (mask) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 2>(p, stream);
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 2>(p, stream);

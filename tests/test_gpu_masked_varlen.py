@@ -226,3 +226,64 @@ def test_key_padding_mask_expanded_over_queries(cuda):
     assert view.stride(2) == 0
     out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=view, head_first=True).cpu()
     _check(out, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("per_head", [False, True])
+def test_key_padding_mask_long_sequences(cuda, per_head, dtype):
+    """From 1024 query rows on, a mask row shared by all queries runs on the 8-wave kernel (mask bytes reduced to
+    words of visible keys per tile).  Trailing padding, holes, a random half, a row that hides its first two key tiles,
+    a batch entry without any visible key (zeros); key count off the tile size, mask rows at odd addresses."""
+    import mindiesd
+    b, n, sq, skv = 5, 2, 1100, 1355
+    q, k, v = _rand((b, n, sq, 128), 41, dtype), _rand((b, n, skv, 128), 42, dtype), _rand((b, n, skv, 128), 43, dtype)
+    g = torch.Generator().manual_seed(44)
+    keep = torch.ones(b, n if per_head else 1, 1, skv, dtype=torch.bool)
+    keep[0, ..., 1000:] = False                       # trailing padding
+    keep[1, ..., 17:40] = False                       # holes, one of them a whole tile
+    keep[1, ..., 256:384] = False
+    keep[2] = torch.rand(keep[2].shape, generator=g) > 0.5
+    keep[3, ..., :300] = False                        # the first two tiles hidden
+    keep[4] = False                                   # nothing visible
+    if per_head:
+        keep[0, 1, ..., 500:] = False
+    full = keep.expand(b, n, sq, skv)
+    ref = attention_math(q, k, v, full, head_first=True)
+    ref[4] = 0
+    view = keep.to(cuda).expand(b, keep.shape[1], sq, skv)
+    assert view.stride(2) == 0
+    out, lse = mindiesd.layers.flash_attn.hip_flash_attn.flash_attention(
+        q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", attn_mask=view, return_lse=True)
+    out = out.cpu()
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3
+    _check(out[:4], ref[:4], max_abs=tol)
+    assert not out[4].any()
+    s = (q.float() @ k.float().transpose(-1, -2)) * 128 ** -0.5
+    want_lse = torch.logsumexp(s.masked_fill(~full, float("-inf")), dim=-1)
+    assert torch.allclose(lse.cpu()[:4], want_lse[:4], atol=5e-3, rtol=0)
+    assert torch.isinf(lse.cpu()[4]).all()
+    # the materialised mask takes the general kernel: same result up to the summation order
+    out_full = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=full.contiguous().to(cuda),
+                                          head_first=True).cpu()
+    assert (out.float() - out_full.float()).abs().max() <= tol
+
+
+def test_key_padding_mask_first_visible_key_far_below_zero(cuda):
+    """Scores hundreds of units below zero and a mask that hides the first tiles: the reference maximum must come
+    from the first tile that shows a key (fp64 yardstick on the queries as the kernel rounds them)."""
+    import math
+    import mindiesd
+    from oracle.attention import attention_fp64
+    sq, skv = 1024, 1500
+    g = torch.Generator().manual_seed(45)
+    q = (8.0 + 0.5 * torch.randn((1, 2, sq, 128), generator=g)).to(torch.bfloat16)
+    k = (-8.0 + 0.5 * torch.randn((1, 2, skv, 128), generator=g)).to(torch.bfloat16)
+    v = torch.randn((1, 2, skv, 128), generator=g).to(torch.bfloat16)
+    keep = torch.zeros(1, 1, 1, skv, dtype=torch.bool)
+    keep[..., 700:1400] = True
+    out = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=keep.to(cuda).expand(1, 1, sq, skv),
+                                     head_first=True).cpu()
+    qs = (q.float() * (128 ** -0.5 * math.log2(math.e))).to(torch.bfloat16)
+    m2 = keep[0, 0].expand(sq, skv).numpy()
+    for n in range(2):
+        _check(out[0, n], attention_fp64(qs[0, n], k[0, n], v[0, n], math.log(2.0), keep=m2))
