@@ -16,7 +16,7 @@ def attention_forward(query, key, value, attn_mask=None, scale=None, fused=True,
     The output has the layout and dtype of ``query``.
 
     Args:
-        attn_mask: [Sq, Skv] or [B|1, N|1, Sq, Skv], True / non-zero = attend.
+        attn_mask: [Sq|1, Skv] or [B|1, N|1, Sq|1, Skv] (query dimension 1: one row for all queries), True / non-zero = attend.
         scale: float softmax scale, default head_dim ** -0.5.
         fused: True runs the HIP flash-attention kernel, False the unfused torch math.
         kwargs: ``opt_mode`` in {'runtime' (default), 'static', 'manual'}; with 'manual',

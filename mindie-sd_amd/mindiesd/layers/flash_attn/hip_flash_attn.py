@@ -47,7 +47,8 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
     """softmax(scale * Q K^T) V on the GPU.  ``layout`` is 'BNSD' or 'BSND'; the output has the
     input's layout and dtype.  Grouped-query attention is supported (N % N_kv == 0).
 
-    ``attn_mask``: [Sq, Skv] or [B|1, N|1, Sq, Skv], non-zero / True = attend (the reference's fused
+    ``attn_mask``: [Sq|1, Skv] or [B|1, N|1, Sq|1, Skv] (query dimension 1: one row for all queries),
+    non-zero / True = attend (the reference's fused
     wrappers hand the vendor kernel ``~mask.to(torch.bool)``, prompt_flash_attn.py:46-47); ``causal``
     keeps key j for query i iff j <= i + (Skv - Sq).  Rows without any visible key give zeros."""
     _check_qkv(query, key, value)
@@ -77,16 +78,17 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
                 mask = attn_mask
                 if mask.dim() == 2:
                     mask = mask[None, None]
-                if (mask.dim() != 4 or mask.shape[-2:] != (sq, skv) or mask.shape[0] not in (1, b)
-                        or mask.shape[1] not in (1, n)):
-                    raise ParametersInvalid(f"attn_mask must be [Sq, Skv] or [B|1, N|1, Sq, Skv] = [{b}|1, {n}|1, {sq}, {skv}], "
-                                            f"but got {tuple(attn_mask.shape)}.")
+                if (mask.dim() != 4 or mask.shape[-1] != skv or mask.shape[-2] not in (1, sq)
+                        or mask.shape[0] not in (1, b) or mask.shape[1] not in (1, n)):
+                    raise ParametersInvalid(f"attn_mask must be [Sq|1, Skv] or [B|1, N|1, Sq|1, Skv] = "
+                                            f"[{b}|1, {n}|1, {sq}|1, {skv}], but got {tuple(attn_mask.shape)}.")
                 mask = mask.to(device=query.device, dtype=torch.bool)
                 if mask.stride(-1) != 1:
                     mask = mask.contiguous()
                 m_sb = mask.stride(0) if mask.shape[0] > 1 else 0
                 m_sn = mask.stride(1) if mask.shape[1] > 1 else 0
-                m_sq = mask.stride(2) if sq > 1 else skv  # 0 for a mask expanded over the queries
+                # 0 for a mask row shared by all queries (a key-padding mask, given as such or expanded over the queries)
+                m_sq = 0 if mask.shape[2] == 1 and sq > 1 else (mask.stride(2) if sq > 1 else skv)
             rc = _native.lib().mindiesd_flash_attention_general_fwd(
                 query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if lse is not None else None, _native.DTYPE_CODE[query.dtype],

@@ -262,6 +262,9 @@ def test_key_padding_mask_long_sequences(cuda, per_head, dtype):
     want_lse = torch.logsumexp(s.masked_fill(~full, float("-inf")), dim=-1)
     assert torch.allclose(lse.cpu()[:4], want_lse[:4], atol=5e-3, rtol=0)
     assert torch.isinf(lse.cpu()[4]).all()
+    # the same mask without the expansion ([B, N|1, 1, Skv])
+    out_b = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=keep.to(cuda), head_first=True).cpu()
+    assert torch.equal(out_b, out)
     # the materialised mask takes the general kernel: same result up to the summation order
     out_full = mindiesd.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=full.contiguous().to(cuda),
                                           head_first=True).cpu()
