@@ -722,11 +722,30 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   static_assert(!gen || (!PAIR && !GATHER), "general mode: dense tensors in their own order");
   const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
-  const int per_xcd = (total + 7) / 8;
-  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (work >= total) return;
-  int bn = work / q_tiles;
-  int qt = work - bn * q_tiles;
+  int bn, qt;
+  if (GEN == 1 && p.causal) {
+    // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
+    // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
+    // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
+    // heads, and it starts its heavy halves first and its light halves last, the larger ones before the smaller.
+    const int units_per_head = (q_tiles + 1) / 2;
+    const int units = p.B * p.N * units_per_head;
+    const int per_xcd = (units + 7) / 8;
+    const int j = blockIdx.x >> 3;
+    const bool heavy = j < per_xcd;
+    const int unit = (blockIdx.x & 7) * per_xcd + (heavy ? j : 2 * per_xcd - 1 - j);
+    if (unit >= units) return;
+    bn = unit / units_per_head;
+    const int u = unit - bn * units_per_head;
+    qt = heavy ? q_tiles - 1 - u : u;
+    if (!heavy && 2 * u == q_tiles - 1) return;  // odd count: the middle tile is its own partner
+  } else {
+    const int per_xcd = (total + 7) / 8;
+    const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (work >= total) return;
+    bn = work / q_tiles;
+    qt = work - bn * q_tiles;
+  }
   int b, n;
   if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
     n = bn;
@@ -734,7 +753,6 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     if (p.causal) qt = (p.seq_meta[4 * b + 1] + kBM - 1) / kBM - 1 - qt;
     bn = b * p.N + n;
   } else {
-    if (gen && !keymask && p.causal) qt = q_tiles - 1 - qt;  // the tiles with the most visible keys start first
     b = bn / p.N;
     n = bn - b * p.N;
   }
@@ -1126,9 +1144,11 @@ static int launch_fa16(const FaParams& p, hipStream_t stream) {
   auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER, GEN, DPAD>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const int total = GEN == 2 ? p.N * p.packed_tiles
-                             : p.B * p.N * (PAIR ? p.NP : (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32));
-  hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8), dim3(NWAVES * 64), kLds, stream, p);
+  const int q_tiles = (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32);
+  const int total = GEN == 2 ? p.N * p.packed_tiles : p.B * p.N * (PAIR ? p.NP : q_tiles);
+  int grid = ((total + 7) / 8) * 8;
+  if (GEN == 1 && p.causal) grid = 16 * ((p.B * p.N * ((q_tiles + 1) / 2) + 7) / 8);  // per XCD: heavy halves, light halves
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
