@@ -723,11 +723,13 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   int bn, qt;
-  if (GEN == 1 && p.causal) {
+  if (PAIR || (GEN == 1 && p.causal)) {
     // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
     // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
     // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
     // heads, and it starts its heavy halves first and its light halves last, the larger ones before the smaller.
+    // PAIR: the pairs of a head are numbered by descending length of their lists; the unit is pair u with pair
+    // NP - 1 - u.
     const int units_per_head = (q_tiles + 1) / 2;
     const int units = p.B * p.N * units_per_head;
     const int per_xcd = (units + 7) / 8;
@@ -737,8 +739,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     if (unit >= units) return;
     bn = unit / units_per_head;
     const int u = unit - bn * units_per_head;
-    qt = heavy ? q_tiles - 1 - u : u;
-    if (!heavy && 2 * u == q_tiles - 1) return;  // odd count: the middle tile is its own partner
+    qt = (heavy != PAIR) ? q_tiles - 1 - u : u;
+    if (!heavy && 2 * u == q_tiles - 1) return;  // odd count: the middle one is its own partner
   } else {
     const int per_xcd = (total + 7) / 8;
     const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
@@ -1148,6 +1150,7 @@ static int launch_fa16(const FaParams& p, hipStream_t stream) {
   const int total = GEN == 2 ? p.N * p.packed_tiles : p.B * p.N * (PAIR ? p.NP : q_tiles);
   int grid = ((total + 7) / 8) * 8;
   if (GEN == 1 && p.causal) grid = 16 * ((p.B * p.N * ((q_tiles + 1) / 2) + 7) / 8);  // per XCD: heavy halves, light halves
+  if (PAIR) grid = 16 * ((p.B * p.N * ((p.NP + 1) / 2) + 7) / 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
