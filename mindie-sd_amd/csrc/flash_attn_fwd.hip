@@ -723,7 +723,25 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
   const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   int bn, qt;
-  if (PAIR || (GEN == 1 && p.causal)) {
+  // Sequences of unequal length (general mode with a table): workgroups are dealt to the XCDs one by one instead of in
+  // runs - tiles in descending order, the (batch, head) index fastest - so every XCD gets its share of the long ones.
+  bool spread = false;
+  if constexpr (GEN == 1 || GEN == 2) {
+    if (p.seq_meta) spread = seqs_uneven(p.seq_meta, p.B);
+  }
+  if (spread) {
+    const int work = blockIdx.x;
+    if (work >= total) return;
+    if (packed) {  // tile-major: the heads of one tile go to consecutive XCDs
+      qt = work / p.N;
+      bn = work - qt * p.N;
+    } else {
+      const int groups = p.B * p.N;
+      const int t = work / groups;
+      bn = work - t * groups;
+      qt = q_tiles - 1 - t;
+    }
+  } else if (PAIR || (GEN == 1 && p.causal)) {
     // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
     // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
     // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
