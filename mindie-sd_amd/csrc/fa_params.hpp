@@ -79,21 +79,25 @@ __device__ __forceinline__ bool packed_find_tile(const int* seq_meta, int nseq, 
 
 // True when the query counts of the table differ enough (the longest more than 1.25 times the mean of the non-empty
 // ones) that equal numbers of consecutive tiles per XCD would be unequal work; wave-uniform, the same in every wave.
-__device__ __forceinline__ bool seqs_uneven(const int* seq_meta, int nseq) {
+// `tiles`: the number of query tiles of `rows` rows that the sequences have together.
+__device__ __forceinline__ bool seqs_uneven(const int* seq_meta, int nseq, int rows, int& tiles) {
   const int lane = threadIdx.x & 63;
   long long sum = 0;
   int longest = 0, filled = 0;
+  tiles = 0;
   for (int c0 = 0; c0 < nseq; c0 += 64) {
     const int s = c0 + lane;
     const int len = s < nseq ? seq_meta[4 * s + 1] : 0;
-    int acc = len, mx = len;
+    int acc = len, mx = len, tl = (len + rows - 1) / rows;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
       acc += __shfl_xor(acc, d, 64);
       mx = max(mx, __shfl_xor(mx, d, 64));
+      tl += __shfl_xor(tl, d, 64);
     }
     sum += __builtin_amdgcn_readfirstlane(acc);
     longest = max(longest, __builtin_amdgcn_readfirstlane(mx));
+    tiles += __builtin_amdgcn_readfirstlane(tl);
     filled += __popcll(__ballot(len > 0));
   }
   return filled > 1 && 4ll * longest * filled > 5ll * sum;

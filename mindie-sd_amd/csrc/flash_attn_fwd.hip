@@ -720,15 +720,20 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   static_assert(!PAIR || NWAVES == 8, "a pair is two groups of four waves");
   constexpr bool gen = GEN != 0, packed = GEN == 2, keymask = GEN == 3;
   static_assert(!gen || (!PAIR && !GATHER), "general mode: dense tensors in their own order");
-  const int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
-  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
+  int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
   int bn, qt;
   // Sequences of unequal length (general mode with a table): workgroups are dealt to the XCDs one by one instead of in
   // runs - tiles in descending order, the (batch, head) index fastest - so every XCD gets its share of the long ones.
   bool spread = false;
   if constexpr (GEN == 1 || GEN == 2) {
-    if (p.seq_meta) spread = seqs_uneven(p.seq_meta, p.B);
+    if (p.seq_meta) {
+      int real_tiles;
+      spread = seqs_uneven(p.seq_meta, p.B, kBM, real_tiles);
+      // packed numbering: the grid is sized for an upper bound; the tiles that exist are what is dealt out
+      if (packed) q_tiles = min(q_tiles, real_tiles);
+    }
   }
+  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
   if (spread) {
     const int work = blockIdx.x;
     if (work >= total) return;
@@ -762,7 +767,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   } else {
     const int per_xcd = (total + 7) / 8;
     const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (work >= total) return;
+    // (the grid of the packed numbering is sized for more tiles than exist: stay inside this XCD's share)
+    if (work >= total || (int)(blockIdx.x >> 3) >= per_xcd) return;
     bn = work / q_tiles;
     qt = work - bn * q_tiles;
   }
