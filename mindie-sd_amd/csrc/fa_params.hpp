@@ -102,15 +102,114 @@ __device__ __forceinline__ bool seqs_uneven(const int* seq_meta, int nseq, int r
   }
   return filled > 1 && 4ll * longest * filled > 5ll * sum;
 }
+
+// Which tile a workgroup of the 16x16x32 kernels (fa_fwd16_kernel, fa_fwd16_d64_kernel; tiles of `rows` query rows)
+// computes: batch entry b, head n, tile qt of the sequence, bn = b * N + n, the sequence's lengths and first tokens.
+// False: nothing to do.  GEN 0: one sequence per batch entry, consecutive tiles of a head on one XCD (workgroups are
+// dealt round-robin to the 8 XCDs).  GEN 1: p.seq_meta and / or causal.  GEN 2: GEN 1 with the packed numbering of
+// p.packed_tiles.  GEN 3: as GEN 0 (the key mask plays no part here).  PAIR: tiles are the p.NP pairs of a head.
+template <int GEN, bool PAIR>
+__device__ __forceinline__ bool fa16_find_work(const FaParams& p, int rows, int& bn, int& qt, int& b, int& n, int& Sq,
+                                               int& Skv, long long& q_tok0, long long& k_tok0) {
+  constexpr bool packed = GEN == 2;
+  int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + rows - 1) / rows;
+  // Sequences of unequal length (general mode with a table): workgroups are dealt to the XCDs one by one instead of in
+  // runs - tiles in descending order, the (batch, head) index fastest - so every XCD gets its share of the long ones.
+  bool spread = false;
+  if constexpr (GEN == 1 || GEN == 2) {
+    if (p.seq_meta) {
+      int real_tiles;
+      spread = seqs_uneven(p.seq_meta, p.B, rows, real_tiles);
+      // packed numbering: the grid is sized for an upper bound; the tiles that exist are what is dealt out
+      if (packed) q_tiles = min(q_tiles, real_tiles);
+    }
+  }
+  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
+  if (spread) {
+    const int work = blockIdx.x;
+    if (work >= total) return false;
+    if (packed) {  // tile-major: the heads of one tile go to consecutive XCDs
+      qt = work / p.N;
+      bn = work - qt * p.N;
+    } else {
+      const int groups = p.B * p.N;
+      const int t = work / groups;
+      bn = work - t * groups;
+      qt = q_tiles - 1 - t;
+    }
+  } else if (PAIR || (GEN == 1 && p.causal)) {
+    // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
+    // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
+    // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
+    // heads, and it starts its heavy halves first and its light halves last, the larger ones before the smaller.
+    // PAIR: the pairs of a head are numbered by descending length of their lists; the unit is pair u with pair
+    // NP - 1 - u.
+    const int units_per_head = (q_tiles + 1) / 2;
+    const int units = p.B * p.N * units_per_head;
+    const int per_xcd = (units + 7) / 8;
+    const int j = blockIdx.x >> 3;
+    const bool heavy = j < per_xcd;
+    const int unit = (blockIdx.x & 7) * per_xcd + (heavy ? j : 2 * per_xcd - 1 - j);
+    if (unit >= units) return false;
+    bn = unit / units_per_head;
+    const int u = unit - bn * units_per_head;
+    qt = (heavy != PAIR) ? q_tiles - 1 - u : u;
+    if (!heavy && 2 * u == q_tiles - 1) return false;  // odd count: the middle one is its own partner
+  } else {
+    const int per_xcd = (total + 7) / 8;
+    const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    // (the grid of the packed numbering is sized for more tiles than exist: stay inside this XCD's share)
+    if (work >= total || (int)(blockIdx.x >> 3) >= per_xcd) return false;
+    bn = work / q_tiles;
+    qt = work - bn * q_tiles;
+  }
+  if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
+    n = bn;
+    if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt, rows)) return false;
+    if (p.causal) qt = (p.seq_meta[4 * b + 1] + rows - 1) / rows - 1 - qt;
+    bn = b * p.N + n;
+  } else {
+    b = bn / p.N;
+    n = bn - b * p.N;
+  }
+  Sq = p.Sq;
+  Skv = p.Skv;
+  q_tok0 = 0;
+  k_tok0 = 0;
+  if constexpr (GEN == 1 || GEN == 2) {
+    if (p.seq_meta) {
+      const int* meta = p.seq_meta + 4 * b;
+      Sq = meta[1];
+      Skv = meta[3];
+      if (qt * rows >= Sq) return false;  // the grid is sized for the longest sequence
+      q_tok0 = meta[0];
+      k_tok0 = meta[2];
+    }
+  }
+  return true;
+}
+
 #endif
+
+// Grid of the 16x16x32 kernels (fa16_find_work above) for p, tiles of `rows` query rows.
+template <int GEN, bool PAIR>
+inline long long fa16_grid(const FaParams& p, int rows) {
+  const long long q_tiles = (p.Sq + rows - 1) / rows;
+  const long long total = GEN == 2 ? (long long)p.N * p.packed_tiles : (long long)p.B * p.N * (PAIR ? p.NP : q_tiles);
+  if (PAIR) return 16 * (((long long)p.B * p.N * ((p.NP + 1) / 2) + 7) / 8);
+  if (GEN == 1 && p.causal) return 16 * (((long long)p.B * p.N * ((q_tiles + 1) / 2) + 7) / 8);  // per XCD: heavy halves, light halves
+  return (total + 7) / 8 * 8;
+}
 
 // Dense attention for head dims other than 128 (flash_attn_hd.hip): D a multiple of 8, at most 256; all options of
 // the general mode (packed sequences, causal, boolean mask, lse).
 int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream);
 
-// Dense attention at head_dim 64 exactly (flash_attn_d64.hip): no mask, no packed sequences; `supported` is false when
-// a K or V (batch, head) slice does not fit the kernel's 32-bit buffer offsets (the general kernel takes those).
+// Attention at head_dim 64 exactly (flash_attn_d64.hip); `gen` as the GEN of fa_fwd16_kernel: 0 dense, 1 p.seq_meta
+// and / or causal, 2 the same with p.packed_tiles (256-row tiles), 3 a mask row shared by all queries.  `supported`
+// is false when a K or V (batch, head) slice does not fit the kernel's 32-bit buffer offsets (the general kernel
+// takes those).
 bool fa16_d64_supported(const FaParams& p);
-int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream);
+int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen = 0);
 
 }  // namespace msd

@@ -1,4 +1,5 @@
-// Dense flash-attention forward for gfx950 (MI355X) at head_dim 64: bf16/fp16, no mask, one sequence per batch entry.
+// Flash-attention forward for gfx950 (MI355X) at head_dim 64: bf16/fp16; dense, and (from 1024 query rows on) causal,
+// packed variable-length sequences and key-padding masks.
 //
 // head_dim 64 is what the reference's own tests of attention_forward run
 // (tests/layers/flash_attn/test_attn_forward.py:31-169) and what its fused dense ops
@@ -119,7 +120,9 @@ constexpr int kD64TileBytes = kD64BN * kD64RowBytes;  // 16 KiB
 constexpr int kD64Lds = 4 * kD64TileBytes;            // two K and two V stages
 constexpr int kD64Ahead = 3;                          // K operand groups requested ahead of their use
 
-template <int DT>
+// GEN as in fa_fwd16_kernel (flash_attn_fwd.hip): 0 dense; 1 per-sequence lengths (p.seq_meta) and / or causal;
+// 2 the same with the packed tile numbering; 3 a boolean mask row shared by all queries of a (batch, head).
+template <int DT, int GEN = 0>
 __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using namespace d64;
@@ -138,24 +141,17 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   const int c = lane & 15;
   const int g = lane >> 4;
 
-  // consecutive query tiles of one head stay on one XCD (workgroups are dealt round-robin to the 8 XCDs)
-  const int q_tiles = (p.Sq + kBM - 1) / kBM;
-  const int total = p.B * p.N * q_tiles;
-  const int per_xcd = (total + 7) / 8;
-  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (work >= total) return;
-  const int bn = work / q_tiles;
-  const int qt = work - bn * q_tiles;
-  const int b = bn / p.N;
-  const int n = bn - b * p.N;
+  constexpr bool gen = GEN != 0, keymask = GEN == 3;
+  int bn, qt, b, n, Sq, Skv;
+  long long q_tok0, k_tok0;  // general mode: first token of the sequence in packed tensors
+  if (!fa16_find_work<GEN, false>(p, kBM, bn, qt, b, n, Sq, Skv, q_tok0, k_tok0)) return;
   const int nkv = n / (p.N / p.Nkv);
-  const int Sq = p.Sq, Skv = p.Skv;
   const int row0 = qt * kBM + wave * 32;  // first query row of this wave
 
-  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
-  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
-  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
-  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn + q_tok0 * p.q_ss;
+  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn + k_tok0 * p.k_ss;
+  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn + k_tok0 * p.v_ss;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn + q_tok0 * p.o_ss;
 
   // ---- Q^T operand, resident: lane (c, g) holds query 16*nq + c, head_dim 32*ks + 8*g .. +8 --------------
   X8 qf[2][2];
@@ -196,10 +192,11 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   // One instruction moves 8 rows of 128 bytes; a wave issues two per operand and tile (rows 8*wave.. and 64 below:
   // the same swizzles, so one per-lane offset per operand serves both).  Keys past the end of the sequence lie
   // outside the descriptors' range and read as zeros.
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kg, 0, (int)(((long long)(Skv - 1) * p.k_ss + 64) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vg, 0, (int)(((long long)(Skv - 1) * p.v_ss + 64) * 2), 0x00020000);
+  // (a sequence without keys exposes nothing: every row reads as zeros and no tile is computed)
+  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + 64) * 2);
+  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + 64) * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, k_range, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, v_range, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
   int k_voff, v_voff;
   {
@@ -237,15 +234,53 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
                   8 * (c & 3);
   }
 
-  const int tiles = (Skv + BN - 1) / BN;
+  // causal: query i sees keys <= i + causal_shift; the last row of this workgroup bounds the tiles it walks
+  const int causal_shift = Skv - Sq;
+  const bool causal = gen && !keymask && p.causal;  // (with a key mask: neither causal nor per-sequence lengths)
+  const int kv_lim = causal ? max(0, min(Skv, qt * kBM + kBM + causal_shift)) : Skv;
+  const int tiles = (kv_lim + BN - 1) / BN;
   load_tile(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   bool first = true;
 
+  // ---- key mask (GEN 3): words of visible keys of the current tile; bit l of word j = key 4 * l + j ------------
+  // (see fa_fwd16_kernel: the bytes of the next tile are fetched during the second product and reduced to scalar words)
+  unsigned kvis[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  unsigned kraw = 0;  // the lane's four mask bytes of the tile that comes next (lanes 0 .. 31)
+  const unsigned char* mask_g = nullptr;
+  if constexpr (keymask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
+  auto mask_request = [&](int key0) __attribute__((always_inline)) {  // the load only
+    if constexpr (keymask) {
+      kraw = 0;
+      const int k4 = key0 + 4 * (lane & 31);
+      if (key0 + BN <= Skv) {
+        __builtin_memcpy(&kraw, mask_g + k4, 4);  // (any alignment)
+      } else {                                    // the tile that runs past the row: byte by byte, inside the row
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned byte = mask_g[min(k4 + j, Skv - 1)];
+          kraw |= (k4 + j < Skv ? byte : 0u) << (8 * j);
+        }
+      }
+    }
+  };
+  auto mask_reduce = [&]() __attribute__((always_inline)) {  // bytes -> words in scalar registers
+    if constexpr (keymask) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        kvis[j] = (unsigned)__builtin_amdgcn_ballot_w64(lane < 32 && ((kraw >> (8 * j)) & 0xffu) != 0);
+    }
+  };
+  if constexpr (keymask) {
+    if (tiles > 0) mask_request(0);
+    mask_reduce();
+  }
+
   auto tile_step = [&](auto stage_c, const int key0, const int next_key0) {
     constexpr int stage = decltype(stage_c)::value;
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+    const unsigned kv_all = kvis[0] & kvis[1] & kvis[2] & kvis[3];
 
     // ---- S^T = K Q^T: 16 accumulation chains of two; operand reads in groups of 2 key blocks of one 32-wide head_dim
     // step, kAhead groups ahead of the matrix instructions that use them (ring of kAhead + 1) -----------------
@@ -292,9 +327,40 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
           }
     }
 
+    // ---- causal: keys beyond the diagonal (the tiles that cross it for some row of this wave) ------------------
+    if constexpr (gen) {
+      if (causal && key0 + BN - 1 > row0 + causal_shift) {
+        const int lim = row0 + c + causal_shift - key0 - 4 * g;  // visible: 16 * kb + i <= lim (+16 for nq = 1)
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (16 * kb + i > lim) sacc[kb][0][i] = -INFINITY;
+            if (16 * kb + i > lim + 16) sacc[kb][1][i] = -INFINITY;
+          }
+      }
+    }
+
+    // ---- key mask: tiles that hide some of their keys ----------------------------------------------------------
+    if constexpr (keymask) {
+      if (kv_all != 0xffffffffu) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned w = kvis[i] >> g;  // key 16 * kb + 4 * g + i is bit 4 * kb + g of word i
+#pragma unroll
+          for (int kb = 0; kb < 8; ++kb)
+            if (!((w >> (4 * kb)) & 1u)) {
+              sacc[kb][0][i] = -INFINITY;
+              sacc[kb][1][i] = -INFINITY;
+            }
+        }
+      }
+    }
+
     // ---- online softmax (exp2 domain): the reference maximum moves only when some row of the wave exceeds it by
     // more than 2^kTau (or on the first tile), so most tiles rescale nothing -------------------------------------
     X8 pf[2][4];
+    bool seen = !keymask;  // key mask: this tile showed some row of the wave a key (all rows share the mask)
 #pragma unroll
     for (int nq = 0; nq < 2; ++nq) {
       float mx = sacc[0][nq][0];
@@ -302,6 +368,7 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
       for (int kb = 0; kb < 8; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
+      if constexpr (keymask) seen = seen || __builtin_amdgcn_ballot_w64(mx > -INFINITY) != 0;
       // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
       float delta = 0.f, alpha = 1.f;
       int moved = 0;
@@ -341,6 +408,9 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
         dst[2 * db + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(v_lds[db]);
       }
     };
+    if constexpr (keymask) {
+      if (next_key0 >= 0) mask_request(next_key0);  // lands during the second product
+    }
     issue(std::integral_constant<int, 0>{}, vf[0]);
     static_for<4>([&](auto step_c) __attribute__((always_inline)) {
       constexpr int j = decltype(step_c)::value;
@@ -364,8 +434,9 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
         lt[nq] = E::mfma16(ones, pf[nq][j], j == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : lt[nq]);
     });
 
-    first = false;
+    first = first && !seen;  // (without a key mask: false from the first tile on)
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next tile has landed
+    mask_reduce();
     __syncthreads();
   };
   for (int t = 0; t < tiles; t += 2) {
@@ -409,14 +480,14 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
 }
 
 
-template <int DT>
+template <int DT, int GEN>
 static int launch_d64(const FaParams& p, hipStream_t stream) {
-  auto kern = fa_fwd16_d64_kernel<DT>;
+  auto kern = fa_fwd16_d64_kernel<DT, GEN>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kD64Lds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const long long total = (long long)p.B * p.N * ((p.Sq + kD64Waves * 32 - 1) / (kD64Waves * 32));
-  if (total > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kern, dim3((unsigned)((total + 7) / 8 * 8)), dim3(kD64Waves * 64), kD64Lds, stream, p);
+  const long long grid = fa16_grid<GEN, false>(p, kD64Waves * 32);
+  if (grid > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kD64Waves * 64), kD64Lds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
@@ -425,9 +496,15 @@ bool fa16_d64_supported(const FaParams& p) {
   return (long long)p.Skv * p.k_ss * 2 < (1ll << 31) && (long long)p.Skv * p.v_ss * 2 < (1ll << 31);
 }
 
-int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream) {
-  if (!fa16_d64_supported(p)) return MSD_ERR_UNSUPPORTED;
-  return dtype == MSD_DTYPE_BF16 ? launch_d64<MSD_DTYPE_BF16>(p, stream) : launch_d64<MSD_DTYPE_F16>(p, stream);
+int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen) {
+  if (!fa16_d64_supported(p) || gen < 0 || gen > 3) return MSD_ERR_UNSUPPORTED;
+  const bool bf = dtype == MSD_DTYPE_BF16;
+  switch (gen) {
+    case 1: return bf ? launch_d64<MSD_DTYPE_BF16, 1>(p, stream) : launch_d64<MSD_DTYPE_F16, 1>(p, stream);
+    case 2: return bf ? launch_d64<MSD_DTYPE_BF16, 2>(p, stream) : launch_d64<MSD_DTYPE_F16, 2>(p, stream);
+    case 3: return bf ? launch_d64<MSD_DTYPE_BF16, 3>(p, stream) : launch_d64<MSD_DTYPE_F16, 3>(p, stream);
+    default: return bf ? launch_d64<MSD_DTYPE_BF16, 0>(p, stream) : launch_d64<MSD_DTYPE_F16, 0>(p, stream);
+  }
 }
 
 }  // namespace msd

@@ -720,81 +720,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   static_assert(!PAIR || NWAVES == 8, "a pair is two groups of four waves");
   constexpr bool gen = GEN != 0, packed = GEN == 2, keymask = GEN == 3;
   static_assert(!gen || (!PAIR && !GATHER), "general mode: dense tensors in their own order");
-  int q_tiles = PAIR ? p.NP : packed ? p.packed_tiles : (p.Sq + kBM - 1) / kBM;
-  int bn, qt;
-  // Sequences of unequal length (general mode with a table): workgroups are dealt to the XCDs one by one instead of in
-  // runs - tiles in descending order, the (batch, head) index fastest - so every XCD gets its share of the long ones.
-  bool spread = false;
-  if constexpr (GEN == 1 || GEN == 2) {
-    if (p.seq_meta) {
-      int real_tiles;
-      spread = seqs_uneven(p.seq_meta, p.B, kBM, real_tiles);
-      // packed numbering: the grid is sized for an upper bound; the tiles that exist are what is dealt out
-      if (packed) q_tiles = min(q_tiles, real_tiles);
-    }
-  }
-  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
-  if (spread) {
-    const int work = blockIdx.x;
-    if (work >= total) return;
-    if (packed) {  // tile-major: the heads of one tile go to consecutive XCDs
-      qt = work / p.N;
-      bn = work - qt * p.N;
-    } else {
-      const int groups = p.B * p.N;
-      const int t = work / groups;
-      bn = work - t * groups;
-      qt = q_tiles - 1 - t;
-    }
-  } else if (PAIR || (GEN == 1 && p.causal)) {
-    // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
-    // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
-    // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
-    // heads, and it starts its heavy halves first and its light halves last, the larger ones before the smaller.
-    // PAIR: the pairs of a head are numbered by descending length of their lists; the unit is pair u with pair
-    // NP - 1 - u.
-    const int units_per_head = (q_tiles + 1) / 2;
-    const int units = p.B * p.N * units_per_head;
-    const int per_xcd = (units + 7) / 8;
-    const int j = blockIdx.x >> 3;
-    const bool heavy = j < per_xcd;
-    const int unit = (blockIdx.x & 7) * per_xcd + (heavy ? j : 2 * per_xcd - 1 - j);
-    if (unit >= units) return;
-    bn = unit / units_per_head;
-    const int u = unit - bn * units_per_head;
-    qt = (heavy != PAIR) ? q_tiles - 1 - u : u;
-    if (!heavy && 2 * u == q_tiles - 1) return;  // odd count: the middle one is its own partner
-  } else {
-    const int per_xcd = (total + 7) / 8;
-    const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    // (the grid of the packed numbering is sized for more tiles than exist: stay inside this XCD's share)
-    if (work >= total || (int)(blockIdx.x >> 3) >= per_xcd) return;
-    bn = work / q_tiles;
-    qt = work - bn * q_tiles;
-  }
-  int b, n;
-  if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
-    n = bn;
-    if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt, kBM)) return;
-    if (p.causal) qt = (p.seq_meta[4 * b + 1] + kBM - 1) / kBM - 1 - qt;
-    bn = b * p.N + n;
-  } else {
-    b = bn / p.N;
-    n = bn - b * p.N;
-  }
+  int bn, qt, b, n, Sq, Skv;
+  long long q_tok0, k_tok0;  // general mode: first token of the sequence in packed tensors
+  if (!fa16_find_work<GEN, PAIR>(p, kBM, bn, qt, b, n, Sq, Skv, q_tok0, k_tok0)) return;
   const int nkv = n / (p.N / p.Nkv);
-  int Sq = p.Sq, Skv = p.Skv;
-  long long q_tok0 = 0, k_tok0 = 0;  // general mode: first token of the sequence in packed tensors
-  if constexpr (gen && !keymask) {
-    if (p.seq_meta) {
-      const int* meta = p.seq_meta + 4 * b;
-      Sq = meta[1];
-      Skv = meta[3];
-      if (qt * kBM >= Sq) return;  // the grid is sized for the longest sequence
-      q_tok0 = meta[0];
-      k_tok0 = meta[2];
-    }
-  }
   // first query row of this wave; rows at or beyond row_end do not exist (tail of the sequence / of the block)
   int row0 = qt * kBM + wave * 32, row_end = Sq;
   if constexpr (PAIR) {
@@ -1170,12 +1099,9 @@ static int launch_fa16(const FaParams& p, hipStream_t stream) {
   auto kern = fa_fwd16_kernel<DT, NWAVES, PAIR, GATHER, GEN, DPAD>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const int q_tiles = (p.Sq + NWAVES * 32 - 1) / (NWAVES * 32);
-  const int total = GEN == 2 ? p.N * p.packed_tiles : p.B * p.N * (PAIR ? p.NP : q_tiles);
-  int grid = ((total + 7) / 8) * 8;
-  if (GEN == 1 && p.causal) grid = 16 * ((p.B * p.N * ((q_tiles + 1) / 2) + 7) / 8);  // per XCD: heavy halves, light halves
-  if (PAIR) grid = 16 * ((p.B * p.N * ((p.NP + 1) / 2) + 7) / 8);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), kLds, stream, p);
+  const long long grid = fa16_grid<GEN, PAIR>(p, NWAVES * 32);
+  if (grid > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NWAVES * 64), kLds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
@@ -1441,8 +1367,13 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
   p.seq_meta = seq_meta; p.causal = causal ? 1 : 0;
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
+  // one mask row for all queries, no other option: the key-mask instantiations of the 16x16x32 kernels
+  const bool key_mask = mask && m_sq == 0 && !causal && !seq_meta;
+  const bool long_rows = Sq >= kGen16MinRows && Skv > kShortKv;
+  if (D == 64 && long_rows && (!mask || key_mask) && fa16_d64_supported(p))
+    return launch_fa16_d64(p, dtype, stream, key_mask ? 3 : 1);
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
-  if (mask && m_sq == 0 && !causal && !seq_meta && Sq >= kGen16MinRows && Skv > kShortKv) {  // one mask row for all queries: the 8-wave kernel
+  if (key_mask && long_rows) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 3>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 3>(p, stream);
   }
@@ -1452,7 +1383,7 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   }
   // Without a mask, long sequences run on the 16x16x32 kernel's general instantiation (256-row tiles); short ones
   // fill the chip better with the 128-row tiles of the 4-wave kernel.
-  if (Sq >= kGen16MinRows && Skv > kShortKv) {
+  if (long_rows) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 1>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 1>(p, stream);
   }
@@ -1493,9 +1424,14 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
   const long long tiles = ((long long)total_q + 127) / 128 + B;
   if (tiles * N > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   p.packed_tiles = (int)tiles;
+  // long sequences on average: the 8-wave kernels, whose tiles are 256 rows
+  const bool long_rows = total_q / B >= kGen16MinRows && total_k / B > kShortKv;
+  if (D == 64 && long_rows && fa16_d64_supported(p)) {
+    p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
+    return launch_fa16_d64(p, dtype, stream, 2);
+  }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
-  // long sequences on average: the 8-wave kernel, whose tiles are 256 rows
-  if (total_q / B >= kGen16MinRows && total_k / B > kShortKv) {
+  if (long_rows) {
     p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 2>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 2>(p, stream);

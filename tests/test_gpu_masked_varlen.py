@@ -93,6 +93,25 @@ def test_causal_bottom_right(cuda, sq, skv):
     assert torch.isinf(lse.cpu()[:, :, ~seen]).all()
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("sq,skv", [(1100, 1100), (1300, 1800), (1800, 1300), (2049, 2049)])
+def test_causal_long_sequences_both_head_dims(cuda, sq, skv, d):
+    """The causal instantiations of the two 16x16x32 kernels (head_dim 128 and 64), three heads (heavy and light
+    tiles are dealt to the XCDs in pairs: an odd and an even tile count)."""
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    q, k, v = _rand((2, 3, sq, d), 8), _rand((2, 3, skv, d), 9), _rand((2, 3, skv, d), 10)
+    out, lse = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BNSD", return_lse=True, causal=True)
+    keep = causal_keep_mask(sq, skv)
+    ref = attention_math(q, k, v, keep, d ** -0.5, head_first=True)
+    seen = keep.any(-1)
+    ref = torch.where(seen[None, None, :, None], ref, torch.zeros((), dtype=ref.dtype))
+    _check(out.cpu(), ref)
+    assert not out.cpu()[:, :, ~seen].any()
+    s = (q.float() @ k.float().transpose(-1, -2)) * d ** -0.5
+    want_lse = torch.logsumexp(s.masked_fill(~keep, float("-inf")), dim=-1)
+    assert torch.allclose(lse.cpu()[:, :, seen], want_lse[:, :, seen], atol=5e-3, rtol=0)
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_forward_varlen(cuda, causal):
     import mindiesd
@@ -150,9 +169,10 @@ def test_varlen_many_sequences_device_table(cuda, d, causal):
     _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_varlen_long_sequences(cuda, causal, dtype):
+def test_varlen_long_sequences(cuda, causal, dtype, d):
     """Sequences of 1024 query tokens and more take the 8-wave kernel (256-row tiles): lengths around the tile edges,
     key counts above and below the query counts (causal rows without any visible key give zeros), a sequence without
     keys and one without queries, grouped heads.  Host lists size the grid by the longest sequence; device tables
@@ -161,8 +181,8 @@ def test_varlen_long_sequences(cuda, causal, dtype):
     lens_q, lens_k = [1500, 1, 0, 1100, 300, 40, 1281], [1500, 700, 5, 1300, 2000, 0, 1000]
     cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
     cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
-    q, k, v = (_rand((sum(lens_q), 4, 128), 31, dtype), _rand((sum(lens_k), 2, 128), 32, dtype),
-               _rand((sum(lens_k), 2, 128), 33, dtype))
+    q, k, v = (_rand((sum(lens_q), 4, d), 31, dtype), _rand((sum(lens_k), 2, d), 32, dtype),
+               _rand((sum(lens_k), 2, d), 33, dtype))
     ref = attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal)
     dev = [t.to(cuda) for t in (q, k, v)]
     out = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
@@ -173,8 +193,8 @@ def test_varlen_long_sequences(cuda, causal, dtype):
     lq2, lk2 = [1500, 1100, 1281, 2049], [1500, 1300, 1000, 2049]
     cq2 = torch.tensor([0] + lq2).cumsum(0).to(torch.int32)
     ck2 = torch.tensor([0] + lk2).cumsum(0).to(torch.int32)
-    q2, k2, v2 = (_rand((sum(lq2), 4, 128), 34, dtype), _rand((sum(lk2), 2, 128), 35, dtype),
-                  _rand((sum(lk2), 2, 128), 36, dtype))
+    q2, k2, v2 = (_rand((sum(lq2), 4, d), 34, dtype), _rand((sum(lk2), 2, d), 35, dtype),
+                  _rand((sum(lk2), 2, d), 36, dtype))
     dev2 = [t.to(cuda) for t in (q2, k2, v2)]
     out_dev = mindiesd.attention_forward_varlen(*dev2, cq2.to(cuda), ck2.to(cuda), causal=causal).cpu()
     out_host = mindiesd.attention_forward_varlen(*dev2, cq2.tolist(), ck2.tolist(), causal=causal).cpu()
@@ -228,15 +248,16 @@ def test_key_padding_mask_expanded_over_queries(cuda):
     _check(out, ref)
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("per_head", [False, True])
-def test_key_padding_mask_long_sequences(cuda, per_head, dtype):
+def test_key_padding_mask_long_sequences(cuda, per_head, dtype, d):
     """From 1024 query rows on, a mask row shared by all queries runs on the 8-wave kernel (mask bytes reduced to
     words of visible keys per tile).  Trailing padding, holes, a random half, a row that hides its first two key tiles,
     a batch entry without any visible key (zeros); key count off the tile size, mask rows at odd addresses."""
     import mindiesd
     b, n, sq, skv = 5, 2, 1100, 1355
-    q, k, v = _rand((b, n, sq, 128), 41, dtype), _rand((b, n, skv, 128), 42, dtype), _rand((b, n, skv, 128), 43, dtype)
+    q, k, v = _rand((b, n, sq, d), 41, dtype), _rand((b, n, skv, d), 42, dtype), _rand((b, n, skv, d), 43, dtype)
     g = torch.Generator().manual_seed(44)
     keep = torch.ones(b, n if per_head else 1, 1, skv, dtype=torch.bool)
     keep[0, ..., 1000:] = False                       # trailing padding
@@ -248,17 +269,17 @@ def test_key_padding_mask_long_sequences(cuda, per_head, dtype):
     if per_head:
         keep[0, 1, ..., 500:] = False
     full = keep.expand(b, n, sq, skv)
-    ref = attention_math(q, k, v, full, head_first=True)
+    ref = attention_math(q, k, v, full, d ** -0.5, head_first=True)
     ref[4] = 0
     view = keep.to(cuda).expand(b, keep.shape[1], sq, skv)
     assert view.stride(2) == 0
     out, lse = mindiesd.layers.flash_attn.hip_flash_attn.flash_attention(
-        q.to(cuda), k.to(cuda), v.to(cuda), 128 ** -0.5, "BNSD", attn_mask=view, return_lse=True)
+        q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BNSD", attn_mask=view, return_lse=True)
     out = out.cpu()
     tol = 2e-2 if dtype == torch.bfloat16 else 2e-3
     _check(out[:4], ref[:4], max_abs=tol)
     assert not out[4].any()
-    s = (q.float() @ k.float().transpose(-1, -2)) * 128 ** -0.5
+    s = (q.float() @ k.float().transpose(-1, -2)) * d ** -0.5
     want_lse = torch.logsumexp(s.masked_fill(~full, float("-inf")), dim=-1)
     assert torch.allclose(lse.cpu()[:4], want_lse[:4], atol=5e-3, rtol=0)
     assert torch.isinf(lse.cpu()[4]).all()
