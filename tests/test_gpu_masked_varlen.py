@@ -202,6 +202,31 @@ def test_varlen_long_sequences(cuda, causal, dtype, d):
     _check(out_dev, attention_varlen(q2, k2, v2, cq2.tolist(), ck2.tolist(), causal=causal))
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_many_long_sequences_device_table(cuda, d, causal):
+    """70 sequences (more than one wave's worth of table entries) of 1024 tokens and more on average, two of them
+    empty and one much longer than the rest, cu_seqlens on the device: the packed numbering of the 8-wave kernels."""
+    import random
+    import mindiesd
+    r = random.Random(100 + d + causal)
+    lens_q = [r.choice([1024, 1100, 1281, 1536]) for _ in range(70)]
+    lens_q[3] = 0
+    lens_q[66] = 0
+    lens_q[40] = 5000
+    lens_k = [max(1, l + r.choice([-300, 0, 0, 257])) for l in lens_q]
+    cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+    cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+    # (values of 0.5 * N(0, 1): a causal row's first keys give outputs that are single value rows, and above 2 one bf16
+    # step is 2^-6, most of the tolerance)
+    q, k, v = _rand((sum(lens_q), 2, d), 81), _rand((sum(lens_k), 1, d), 82), _rand((sum(lens_k), 1, d), 83, mul=0.5)
+    dev = [t.to(cuda) for t in (q, k, v)]
+    out_dev = mindiesd.attention_forward_varlen(*dev, cu_q.to(cuda), cu_k.to(cuda), causal=causal).cpu()
+    out_host = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
+    assert torch.equal(out_dev, out_host)
+    _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
+
+
 def test_varlen_single_sequence_equals_dense(cuda):
     import mindiesd
     q, k, v = _rand((700, 2, 128), 14, mul=0.5), _rand((700, 2, 128), 15, mul=0.5), _rand((700, 2, 128), 16, mul=0.5)
