@@ -179,7 +179,7 @@ def extra_dense_1p3b(device, steps, warmup):
 
 def extra_head_dims(device, steps, warmup):
     """Dense attention at head dims other than 128 at a 17776-token sequence: 64 (its own kernel), 72 and 96 (computed
-    as head_dim 128 on the dense kernel) and 256 (the general kernel)."""
+    as head_dim 128 on the dense kernel) and 256 (its own kernel of the same design)."""
     import torch
     import mindiesd
     res = {"workload": "dense bf16 B1 S17776 (13x30x45 latent tokens + 226 text tokens), N48 D64 / N48 D72 / N32 D96 / N12 D256"}

@@ -162,6 +162,37 @@ def test_head_dims_between_64_and_128_on_the_dense_kernel(cuda, d, sq, skv, dtyp
     assert torch.equal(out_c, out)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [136, 160, 192, 248, 256])
+@pytest.mark.parametrize("sq,skv", [(2311, 3001), (33, 4100), (600, 385)])
+def test_head_dims_above_128_on_their_dense_kernel(cuda, d, sq, skv, dtype):
+    """Dense attention without a mask at head dims above 128 runs on a kernel of the 128-wide design with 512-byte rows
+    (csrc/flash_attn_d256.hip; widths below 256 are computed as 256); an all-true mask sends the same inputs through
+    the general kernel.  q, k, v are views of 256-wide buffers whose columns past the head_dim hold NaN: nothing
+    beyond a row's own elements may reach the result.  Grouped-query heads, BSND storage."""
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    def in_nan_buffer(t):
+        buf = torch.full(t.shape[:-1] + (256,), float("nan"), dtype=t.dtype, device=cuda)
+        buf[..., :d] = t.to(cuda)
+        return buf[..., :d]
+    q, k, v = _rand((1, sq, 4, d), 90, dtype), _rand((1, skv, 2, d), 91, dtype), _rand((1, skv, 2, d), 92, dtype)
+    dq, dk, dv = in_nan_buffer(q), in_nan_buffer(k), in_nan_buffer(v)
+    out, lse = flash_attention(dq, dk, dv, d ** -0.5, "BSND", return_lse=True)
+    assert not torch.isnan(out.float()).any()
+    gen, lse_g = flash_attention(dq, dk, dv, d ** -0.5, "BSND", return_lse=True,
+                                 attn_mask=torch.ones(sq, skv, dtype=torch.bool, device=cuda))
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3
+    assert (out.float() - gen.float()).abs().max().item() <= tol
+    # (both sums are taken over probabilities rounded to 16 bits against different reference maxima: 64- and 32-key tiles)
+    assert (lse - lse_g).abs().max().item() < 3e-3
+    rows = sorted({0, 1, 15, 16, 31, 32, sq // 2, sq - 2, sq - 1} & set(range(sq)))
+    kk, vv = k.repeat_interleave(2, dim=2), v.repeat_interleave(2, dim=2)
+    ref = attention_math(q[:, rows], kk, vv, None, d ** -0.5, head_first=False)
+    _check(out[:, rows].cpu(), ref, max_abs=tol, min_cos=0.9999 if dtype == torch.bfloat16 else 0.99999)
+    out_c = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BSND")
+    assert torch.equal(out_c, out)
+
+
 def test_rejected_head_dims(cuda):
     import mindiesd
     from mindiesd.utils.exception import ParametersInvalid
