@@ -122,7 +122,10 @@ constexpr int kD64Ahead = 3;                          // K operand groups reques
 
 // GEN as in fa_fwd16_kernel (flash_attn_fwd.hip): 0 dense; 1 per-sequence lengths (p.seq_meta) and / or causal;
 // 2 the same with the packed tile numbering; 3 a boolean mask row shared by all queries of a (batch, head).
-template <int DT, int GEN = 0>
+// DPAD (dense only): head dims below 64 (p.head_dim, a multiple of 8) computed as 64: the query operand is zero from
+// the real head_dim on, the lanes that would stage the 16-byte chunks of K and V past it request an offset beyond
+// the buffers' range (the DMA writes zeros for them without touching memory), output columns past it are not stored.
+template <int DT, int GEN = 0, bool DPAD = false>
 __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using namespace d64;
@@ -142,6 +145,8 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   const int g = lane >> 4;
 
   constexpr bool gen = GEN != 0, keymask = GEN == 3;
+  static_assert(!DPAD || !gen, "padded head dims: dense only");
+  const int hd = DPAD ? p.head_dim : 64;
   int bn, qt, b, n, Sq, Skv;
   long long q_tok0, k_tok0;  // general mode: first token of the sequence in packed tensors
   if (!fa16_find_work<GEN, false>(p, kBM, bn, qt, b, n, Sq, Skv, q_tok0, k_tok0)) return;
@@ -162,8 +167,8 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
     const T* src = qg + (long long)(ok ? qrow : 0) * p.q_ss + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      X8 v = *(const X8*)(src + 32 * ks);
-      if (!ok) v = X8{0};
+      const bool in = ok && (!DPAD || 32 * ks + 8 * g < hd);  // (a chunk of 8 lies wholly inside or outside)
+      X8 v = in ? *(const X8*)(src + 32 * ks) : X8{0};
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = E::from_float((float)v[j] * p.scale_log2);
       qf[nq][ks] = v;
@@ -193,8 +198,8 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   // the same swizzles, so one per-lane offset per operand serves both).  Keys past the end of the sequence lie
   // outside the descriptors' range and read as zeros.
   // (a sequence without keys exposes nothing: every row reads as zeros and no tile is computed)
-  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + 64) * 2);
-  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + 64) * 2);
+  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + hd) * 2);
+  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + hd) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, k_range, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, v_range, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
@@ -202,8 +207,13 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   {
     const int row = 8 * wave + (lane >> 3);
     const int pc = lane & 7;  // physical 16-byte chunk this lane fills
-    k_voff = row * k_row_bytes + ((pc ^ ((row >> 1) & 7)) << 4);
-    v_voff = row * v_row_bytes + (((((pc >> 1) ^ ((row >> 1) & 3)) << 1) | (pc & 1)) << 4);
+    const int kc = pc ^ ((row >> 1) & 7), vc = (((pc >> 1) ^ ((row >> 1) & 3)) << 1) | (pc & 1);  // logical chunks
+    k_voff = row * k_row_bytes + (kc << 4);
+    v_voff = row * v_row_bytes + (vc << 4);
+    if constexpr (DPAD) {  // chunks past the head_dim: an offset beyond every range
+      if (kc * 8 >= hd) k_voff = 0x7ffffff0;
+      if (vc * 8 >= hd) v_voff = 0x7ffffff0;
+    }
   }
   auto load_tile = [&](int key0, int stage) {
     MSD_LDS char* kb = smem + stage * kTileBytes;
@@ -471,7 +481,7 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
     // rows are padded by 8 bytes, so a 16-byte chunk is read as two 8-byte halves
     const i32x2_t lo = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c8 * 16);
     const i32x2_t hi = *(MSD_LDS const i32x2_t*)(ost + row * kORowBytes + c8 * 16 + 8);
-    if (qrow < Sq) {
+    if (qrow < Sq && (!DPAD || c8 * 8 < hd)) {
       i32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
       *(i32x4_t*)(og + (long long)qrow * p.o_ss + c8 * 8) = v;
     }
@@ -480,9 +490,9 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
 }
 
 
-template <int DT, int GEN>
+template <int DT, int GEN, bool DPAD = false>
 static int launch_d64(const FaParams& p, hipStream_t stream) {
-  auto kern = fa_fwd16_d64_kernel<DT, GEN>;
+  auto kern = fa_fwd16_d64_kernel<DT, GEN, DPAD>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kD64Lds) != hipSuccess)
     return MSD_ERR_LAUNCH;
   const long long grid = fa16_grid<GEN, false>(p, kD64Waves * 32);
@@ -492,8 +502,17 @@ static int launch_d64(const FaParams& p, hipStream_t stream) {
 }
 
 bool fa16_d64_supported(const FaParams& p) {
-  // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
-  return (long long)p.Skv * p.k_ss * 2 < (1ll << 31) && (long long)p.Skv * p.v_ss * 2 < (1ll << 31);
+  // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base, below the offset that stands
+  // for "no data"
+  return (long long)p.Skv * p.k_ss * 2 < 0x7fffff00ll && (long long)p.Skv * p.v_ss * 2 < 0x7fffff00ll;
+}
+
+int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream) {
+  if (!fa16_d64_supported(p) || D <= 0 || D >= 64 || (D & 7)) return MSD_ERR_UNSUPPORTED;
+  FaParams pp = p;
+  pp.head_dim = D;
+  return dtype == MSD_DTYPE_BF16 ? launch_d64<MSD_DTYPE_BF16, 0, true>(pp, stream)
+                                 : launch_d64<MSD_DTYPE_F16, 0, true>(pp, stream);
 }
 
 int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen) {

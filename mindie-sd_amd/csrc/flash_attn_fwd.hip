@@ -1287,6 +1287,7 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 0, true>(p, stream);
   }
   if (D > 128 && Skv > kShortKv && fa16_d256_supported(p)) return launch_fa16_d256(p, dtype, D, stream);
+  if (D < 64 && Skv > kShortKv && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream);
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   // A few key tiles per query tile (cross attention over a short text): the launch is mostly reading Q and writing O,
   // and two 4-wave workgroups per CU overlap one's memory phases with the other's tiles better than one 8-wave

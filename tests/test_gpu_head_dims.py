@@ -133,15 +133,16 @@ def test_head_dim_64_dense_kernel_against_general_kernel_and_oracle(cuda, sq, sk
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("d", [72, 88, 96, 120])
+@pytest.mark.parametrize("d", [8, 40, 56, 72, 88, 96, 120])
 @pytest.mark.parametrize("sq,skv", [(2311, 3001), (33, 4100), (600, 385)])
-def test_head_dims_between_64_and_128_on_the_dense_kernel(cuda, d, sq, skv, dtype):
-    """Dense attention without a mask at these head dims runs as head_dim 128 on the 16x16x32 kernel; an all-true mask
-    sends the same inputs through the general kernel.  q, k, v are views of 128-wide buffers whose columns past the
-    head_dim hold NaN: nothing beyond a row's own elements may reach the result.  Grouped-query heads, BSND storage."""
+def test_head_dims_below_128_on_the_dense_kernels(cuda, d, sq, skv, dtype):
+    """Dense attention without a mask at these head dims runs as head_dim 64 (below 64) or 128 (above) on the 16x16x32
+    kernels; an all-true mask sends the same inputs through the general kernel.  q, k, v are views of 64- / 128-wide
+    buffers whose columns past the head_dim hold NaN: nothing beyond a row's own elements may reach the result.
+    Grouped-query heads, BSND storage."""
     from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
     def in_nan_buffer(t):
-        buf = torch.full(t.shape[:-1] + (128,), float("nan"), dtype=t.dtype, device=cuda)
+        buf = torch.full(t.shape[:-1] + (64 if d < 64 else 128,), float("nan"), dtype=t.dtype, device=cuda)
         buf[..., :d] = t.to(cuda)
         return buf[..., :d]
     q, k, v = _rand((1, sq, 6, d), 70, dtype), _rand((1, skv, 2, d), 71, dtype), _rand((1, skv, 2, d), 72, dtype)
