@@ -49,7 +49,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 constexpr int kD256Waves = 8, kD256BN = 64, kD256RowBytes = 512;
 constexpr int kD256TileBytes = kD256BN * kD256RowBytes;  // 32 KiB
 constexpr int kD256Lds = 4 * kD256TileBytes;              // two K and two V stages
-constexpr int kD256Ahead = 3;                             // K operand groups requested ahead of their use
+#ifndef FA16_D256_AHEAD
+#define FA16_D256_AHEAD 3
+#endif
+constexpr int kD256Ahead = FA16_D256_AHEAD;               // K operand groups requested ahead of their use
 
 template <int DT, bool DPAD>
 __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const FaParams p) {
