@@ -2,6 +2,7 @@
 // (other head dims).
 #pragma once
 #include "common.hpp"
+#include "fa16_work.hpp"
 
 namespace msd {
 
@@ -124,45 +125,16 @@ __device__ __forceinline__ bool fa16_find_work(const FaParams& p, int rows, int&
       if (packed) q_tiles = min(q_tiles, real_tiles);
     }
   }
-  const int total = (packed ? 1 : p.B) * p.N * q_tiles;
-  if (spread) {
-    const int work = blockIdx.x;
-    if (work >= total) return false;
-    if (packed) {  // tile-major: the heads of one tile go to consecutive XCDs
-      qt = work / p.N;
-      bn = work - qt * p.N;
-    } else {
-      const int groups = p.B * p.N;
-      const int t = work / groups;
-      bn = work - t * groups;
-      qt = q_tiles - 1 - t;
-    }
-  } else if (PAIR || (GEN == 1 && p.causal)) {
-    // Causal: tile t of a head has t + 1 tiles' worth of keys, so equal counts of consecutive tiles per XCD are not
-    // equal work (12 heads on 8 XCDs: 1.75 against 1.25 heads' worth).  The unit that is dealt out is tile
-    // q_tiles - 1 - u together with tile u: units weigh the same, an XCD still gets consecutive units of the same
-    // heads, and it starts its heavy halves first and its light halves last, the larger ones before the smaller.
-    // PAIR: the pairs of a head are numbered by descending length of their lists; the unit is pair u with pair
-    // NP - 1 - u.
-    const int units_per_head = (q_tiles + 1) / 2;
-    const int units = p.B * p.N * units_per_head;
-    const int per_xcd = (units + 7) / 8;
-    const int j = blockIdx.x >> 3;
-    const bool heavy = j < per_xcd;
-    const int unit = (blockIdx.x & 7) * per_xcd + (heavy ? j : 2 * per_xcd - 1 - j);
-    if (unit >= units) return false;
-    bn = unit / units_per_head;
-    const int u = unit - bn * units_per_head;
-    qt = (heavy != PAIR) ? q_tiles - 1 - u : u;
-    if (!heavy && 2 * u == q_tiles - 1) return false;  // odd count: the middle one is its own partner
-  } else {
-    const int per_xcd = (total + 7) / 8;
-    const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    // (the grid of the packed numbering is sized for more tiles than exist: stay inside this XCD's share)
-    if (work >= total || (int)(blockIdx.x >> 3) >= per_xcd) return false;
-    bn = work / q_tiles;
-    qt = work - bn * q_tiles;
-  }
+  // (fa16_work.hpp: runs of consecutive tiles per XCD; units of a heavy and a light tile - causal: tile t of a head has
+  // t + 1 tiles' worth of keys, PAIR: the pairs of a head are numbered by descending length of their lists - so that
+  // 12 heads on 8 XCDs are not 1.75 against 1.25 heads' worth of work; or one by one)
+  const int groups = (packed ? 1 : p.B) * p.N;
+  const fa16::Work w = spread ? fa16::spread(blockIdx.x, groups, q_tiles, packed)
+                       : (PAIR || (GEN == 1 && p.causal)) ? fa16::units(blockIdx.x, groups, q_tiles, PAIR)
+                                                           : fa16::runs(blockIdx.x, groups, q_tiles);
+  if (w.group < 0) return false;
+  bn = w.group;
+  qt = w.tile;
   if constexpr (packed) {  // bn is the head; the tile's sequence comes from the table
     n = bn;
     if (!packed_find_tile(p.seq_meta, p.B, qt, b, qt, rows)) return false;
@@ -194,11 +166,10 @@ __device__ __forceinline__ bool fa16_find_work(const FaParams& p, int rows, int&
 // Grid of the 16x16x32 kernels (fa16_find_work above) for p, tiles of `rows` query rows.
 template <int GEN, bool PAIR>
 inline long long fa16_grid(const FaParams& p, int rows) {
-  const long long q_tiles = (p.Sq + rows - 1) / rows;
-  const long long total = GEN == 2 ? (long long)p.N * p.packed_tiles : (long long)p.B * p.N * (PAIR ? p.NP : q_tiles);
-  if (PAIR) return 16 * (((long long)p.B * p.N * ((p.NP + 1) / 2) + 7) / 8);
-  if (GEN == 1 && p.causal) return 16 * (((long long)p.B * p.N * ((q_tiles + 1) / 2) + 7) / 8);  // per XCD: heavy halves, light halves
-  return (total + 7) / 8 * 8;
+  const long long tiles = PAIR ? p.NP : GEN == 2 ? p.packed_tiles : (p.Sq + rows - 1) / rows;
+  const long long groups = (GEN == 2 ? 1ll : (long long)p.B) * p.N;
+  if (PAIR || (GEN == 1 && p.causal)) return fa16::units_grid(groups, tiles);
+  return fa16::runs_grid(groups, tiles);
 }
 
 // Dense attention for head dims other than 128 (flash_attn_hd.hip): D a multiple of 8, at most 256; all options of
