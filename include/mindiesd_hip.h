@@ -147,12 +147,11 @@ int mindiesd_block_sparse_attention_general_fwd(const void* q, const void* k, co
                                                 hipStream_t stream);
 
 /* Block-sparse attention driven by the int8 mask itself (mask [B][N][ceil(Sq/128)][ceil(Skv/128)], non-zero =
- * attend), in two passes over PAIRED query blocks: query blocks of a head whose mask rows overlap most are paired
- * on the device; pass 1 computes, per pair, the key blocks both partners selected with one 256-row workgroup (each
- * K/V tile is fetched once for both, the dense kernel's inner loop); pass 2 adds, per query block, the key blocks
- * only it selected, continuing the running softmax of pass 1.  Same semantics as
- * mindiesd_block_sparse_attention_fwd on the lists of the mask; results differ by the order of the accumulation and
- * by one more rounding to the 16-bit output type (pass 1 hands its normalised rows to pass 2 through `out`), well
+ * attend), over PAIRED query blocks: query blocks of a head whose mask rows overlap most are paired on the device;
+ * one 256-row workgroup per pair first walks the key blocks both partners selected (each K/V tile is fetched once for
+ * both, the dense kernel's inner loop), then each partner's four waves walk the key blocks only it selected, in
+ * 64-key sub-tiles, the running softmax going on.  Same semantics as mindiesd_block_sparse_attention_fwd on the lists
+ * of the mask; results differ by the order of the accumulation only, well
  * inside the reference kernels' 2^-6 rule; replaces the same reference kernels.  token_order (optional, self-attention): as in the gather entry
  * point above.  workspace: mindiesd_block_sparse_attention_paired_workspace_size bytes, 16-byte aligned.
  * Returns 2 when the mask is too large for the pairing kernels (more than 2048 key blocks, or mask rows of one

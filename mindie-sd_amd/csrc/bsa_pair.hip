@@ -4,14 +4,13 @@
 // work - twice the bytes per flop of the dense kernel, whose workgroup shares every K/V tile between 256 query rows -
 // and at DiT sizes that stream (L2 -> LDS, and HBM -> L2 for the tiles the XCD's L2 no longer holds) is what bounds
 // it.  Query blocks that select mostly the same key blocks (in video latents: the same spatial region one frame
-// apart) can share their tiles: they are paired here, and the attention then runs in two passes
-// (flash_attn_fwd.hip): the key blocks both partners selected with one 256-row workgroup per pair at the dense
-// kernel's rate, the rest per query block, continuing the running softmax of the first pass.
+// apart) can share their tiles: they are paired here, and the attention kernel (the PAIR instantiation of
+// fa_fwd16_kernel, flash_attn_fwd.hip) gives every pair one 256-row workgroup: the key blocks both partners selected
+// at the dense kernel's rate, then each partner's own key blocks with its four waves, the running softmax going on.
 //
 // No counterpart in the reference (its sparse kernels are closed vendor binaries behind
 // csrc/plugin/block_sparse_attention.cpp:31-121); the result of the attention does not depend on the pairing
-// except for the order of the floating-point accumulation and for one rounding: the first pass leaves its
-// normalised rows in the 16-bit output tensor, from where the second pass takes them up again.
+// except for the order of the floating-point accumulation.
 //
 // bsa_bits_kernel:       int8 mask rows -> bit rows + their popcounts.
 // bsa_candidates_kernel: per query block the kCand blocks of the same head with the largest similarity

@@ -32,6 +32,8 @@ struct FaParams {
   int NP;
   float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)
   const int* init_cnt;  // second pass: [B * N][QB] key blocks the first pass covered for this query block (0: none)
+  const int* ex_idx;    // PAIR kernel, optional: [B * N][QB][kb_stride] key blocks only this query block selected, walked by
+  const int* ex_cnt;    //   its own four waves after the pair's shared list ([B * N][QB] counts); then no second pass follows
   // general mode (MODE = 1 instantiations only)
   const int* seq_meta;        // optional [B][4]: first query token, query count, first key token, key count of
                               // sequence b inside packed (token, head, dim) tensors; Sq is then the longest count

@@ -1047,6 +1047,177 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
       id_a = id_c;
       id_b = id_d;
     }
+    // ---- second phase (p.ex_idx given): the key blocks that only one partner selected ----------------------------
+    // Each group of four waves walks the list of its own query block in sub-tiles of 64 keys, staged into its own half
+    // of the four LDS buffers by its own waves; the eight waves still meet at one barrier per sub-tile, and the
+    // running softmax simply goes on.  The traffic of these blocks (64 KiB for 128 rows, twice the bytes per flop of
+    // the shared tiles) runs beside other workgroups' shared phases instead of in a launch of its own.
+    if (p.ex_idx) {
+      const int grp = wave >> 2, w4 = wave & 3;
+      constexpr int kHalf = kTileBytes / 2;
+      const long long pair_lin = (long long)bn * p.NP + qt;
+      const int qb_mine = __builtin_amdgcn_readfirstlane(p.pairs[pair_lin * 2 + grp]);
+      const int qb_other = __builtin_amdgcn_readfirstlane(p.pairs[pair_lin * 2 + (grp ^ 1)]);
+      const int* e_ptr = p.ex_idx + ((long long)bn * p.QB + max(qb_mine, 0)) * p.kb_stride;
+      const int e_n = qb_mine >= 0 ? __builtin_amdgcn_readfirstlane(p.ex_cnt[(long long)bn * p.QB + qb_mine]) : 0;
+      const int e_o = qb_other >= 0 ? __builtin_amdgcn_readfirstlane(p.ex_cnt[(long long)bn * p.QB + qb_other]) : 0;
+      const int my_steps = 2 * e_n, steps = 2 * max(e_n, e_o);
+      // this group's halves of the stages; its waves stage rows 4 * w4 + 16 * i of a sub-tile
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) k_lds[ks] += grp * kHalf;
+#pragma unroll
+      for (int db = 0; db < 4; ++db) v_lds[db] += grp * kHalf;
+      k_voff -= 16 * grp * k_row_bytes;
+      v_voff -= 16 * grp * v_row_bytes;
+      auto load_half = [&](int key0, int stage) {
+        MSD_LDS char* kb = smem + stage * kTileBytes + grp * kHalf;
+        MSD_LDS char* vb = smem + (2 + stage) * kTileBytes + grp * kHalf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int g4 = i * 4 + w4;  // 4-row group of the sub-tile
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g4 * 1024), 16, k_voff,
+                                                   (key0 + 16 * i) * k_row_bytes, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g4 * 1024), 16, v_voff,
+                                                   (key0 + 16 * i) * v_row_bytes, 0, 0);
+        }
+      };
+      auto half_step = [&](auto stage_c, const int key0, const int next_key0) {
+        constexpr int stage = decltype(stage_c)::value;
+        if (next_key0 >= 0) load_half(next_key0, stage ^ 1);
+        if (key0 >= 0) {
+          // S^T = K Q^T over 4 key blocks (see tile_step)
+          f32x4_t sacc[4][2];
+          constexpr int kAhead = FA16_AHEAD;
+          X8 afrag[kAhead + 1][2];
+          auto k_read = [&](auto gi_c, X8(&dst)[2]) __attribute__((always_inline)) {
+            constexpr int gi = decltype(gi_c)::value;
+            constexpr int ks = gi >> 1, qu = gi & 1;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+              dst[i] = *(MSD_LDS const X8*)(uintptr_t)(k_lds[ks] + stage * kTileBytes + (2 * qu + i) * 16 * kRowBytes);
+          };
+          static_for<kAhead>([&](auto gi_c) __attribute__((always_inline)) { k_read(gi_c, afrag[decltype(gi_c)::value]); });
+          static_for<8>([&](auto gi_c) __attribute__((always_inline)) {
+            constexpr int gi = decltype(gi_c)::value;
+            constexpr int ks = gi >> 1, qu = gi & 1;
+            if constexpr (gi + kAhead < 8) k_read(std::integral_constant<int, gi + kAhead>{}, afrag[(gi + kAhead) % (kAhead + 1)]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+              for (int nq = 0; nq < 2; ++nq)
+                sacc[2 * qu + i][nq] =
+                    E::mfma16(afrag[gi % (kAhead + 1)][i], qf[nq][ks], ks == 0 ? negm[nq] : sacc[2 * qu + i][nq]);
+          });
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+          for (int gi = 0; gi < 8 - kAhead; ++gi) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (key0 + 64 > Skv) {
+#pragma unroll
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (key0 + 16 * kb + 4 * g + i >= Skv) {
+                  sacc[kb][0][i] = -INFINITY;
+                  sacc[kb][1][i] = -INFINITY;
+                }
+          }
+          X8 pf[2][2];
+#pragma unroll
+          for (int nq = 0; nq < 2; ++nq) {
+            float mx = sacc[0][nq][0];
+#pragma unroll
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][nq][i]);
+            l_run[nq] += lt[nq][0];
+            // (the rare path as plain code: this phase is bound by its memory traffic)
+            if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
+              mx = quarter_max(mx);
+              float delta = first ? mx : fmaxf(mx, 0.f);
+              delta = (delta == -INFINITY) ? 0.f : delta;
+              const float alpha = first ? 1.f : fast_exp2(-delta);
+              l_run[nq] *= alpha;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) negm[nq][i] -= delta;
+#pragma unroll
+              for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sacc[kb][nq][i] -= delta;
+#pragma unroll
+              for (int db = 0; db < 8; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oacc[db][nq][i] *= alpha;
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              X8 pk;
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                pk[t] = E::from_float(fast_exp2(sacc[2 * j][nq][t]));
+                pk[4 + t] = E::from_float(fast_exp2(sacc[2 * j + 1][nq][t]));
+              }
+              pf[nq][j] = pk;
+            }
+          }
+          s16x4_t vf[2][8];
+          auto issue = [&](auto step_c, s16x4_t(&dst)[8]) __attribute__((always_inline)) {
+            constexpr int s = decltype(step_c)::value;
+            constexpr int j = s >> 1, dbh = s & 1;
+            constexpr int off = stage * kTileBytes + 32 * j * kRowBytes;
+#pragma unroll
+            for (int d4 = 0; d4 < 4; ++d4) {
+              const unsigned a = v_lds[d4] ^ (dbh << 7);
+              dst[2 * d4] = lds_read_tr16_async<off>(a);
+              dst[2 * d4 + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(a);
+            }
+          };
+          issue(std::integral_constant<int, 0>{}, vf[0]);
+          static_for<4>([&](auto step_c) __attribute__((always_inline)) {
+            constexpr int s = decltype(step_c)::value;
+            constexpr int j = s >> 1, dbh = s & 1;
+            if constexpr (s + 1 < 4) {
+              issue(std::integral_constant<int, s + 1>{}, vf[(s + 1) & 1]);
+              lds_wait_tr<8>(vf[s & 1]);
+            } else {
+              lds_wait_tr<0>(vf[s & 1]);
+            }
+#pragma unroll
+            for (int d4 = 0; d4 < 4; ++d4) {
+              union { s16x4_t s2[2]; X8 x; } u;
+              u.s2[0] = vf[s & 1][2 * d4];
+              u.s2[1] = vf[s & 1][2 * d4 + 1];
+#pragma unroll
+              for (int nq = 0; nq < 2; ++nq) oacc[4 * dbh + d4][nq] = E::mfma16(u.x, pf[nq][j], oacc[4 * dbh + d4][nq]);
+            }
+            if constexpr (dbh == 0) {
+#pragma unroll
+              for (int nq = 0; nq < 2; ++nq)
+                lt[nq] = E::mfma16(ones, pf[nq][j], j == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : lt[nq]);
+            }
+          });
+          first = false;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next sub-tile has landed
+        __syncthreads();
+      };
+      // key of sub-tile st of this group (-1: past its list); the block ids come by scalar loads one block ahead
+      int e_cur = my_steps > 0 ? __builtin_amdgcn_readfirstlane(e_ptr[0]) : 0;
+      if (my_steps > 0) load_half(e_cur * 128, 0);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      for (int st = 0; st < steps; st += 2) {  // one 128-key block per iteration: its two halves
+        const int e_next = st + 2 < my_steps ? __builtin_amdgcn_readfirstlane(e_ptr[(st >> 1) + 1]) : 0;
+        const bool mine = st < my_steps;
+        half_step(std::integral_constant<int, 0>{}, mine ? e_cur * 128 : -1, mine ? e_cur * 128 + 64 : -1);
+        half_step(std::integral_constant<int, 1>{}, mine ? e_cur * 128 + 64 : -1, st + 2 < my_steps ? e_next * 128 : -1);
+        e_cur = e_next;
+      }
+    }
   } else {
     for (int t = 0; t < tiles; t += 2) {
       tile_step(std::integral_constant<int, 0>{}, t * BN, t + 1 < tiles ? (t + 1) * BN : -1);
@@ -1064,8 +1235,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     if (p.lse && g == 0 && qrow_l < row_end)
       p.lse[((long long)b * p.N + n) * p.Sq + (GATHER ? p.tok[qrow_l] : qrow_l)] =
           l_tot > 0.f ? -negm[nq][0] * 0.6931471805599453f + __logf(l_tot) : -INFINITY;
-    if constexpr (PAIR) {
-      if (g == 0 && qrow_l < row_end)
+    if constexpr (PAIR) {  // (only a second launch would read it)
+      if (!p.ex_idx && g == 0 && qrow_l < row_end)
         p.state[((long long)b * p.N + n) * p.Sq + qrow_l] = l_tot > 0.f ? -negm[nq][0] + __log2f(l_tot) : -INFINITY;
     }
 #pragma unroll
@@ -1250,15 +1421,22 @@ int mindiesd_block_sparse_attention_paired_fwd(const void* q, const void* k, con
   p.tok = token_order;
   p.QB = QB;
   p.state = state;
-  // pass 1: one workgroup per pair over the shared list
+  // one workgroup per pair: the shared list with all eight waves, then each partner's own list with its four
   p.pairs = t.pairs; p.NP = t.NP;
   p.blk_idx = t.sh_idx; p.blk_cnt = t.sh_cnt; p.kb_stride = KB;
+#if !defined(MSD_BSA_TWO_PASS)
+  p.ex_idx = t.ex_idx; p.ex_cnt = t.ex_cnt;
+#endif
   if (dtype == MSD_DTYPE_BF16)
     rc = token_order ? launch_fa16<MSD_DTYPE_BF16, 8, true, true>(p, stream) : launch_fa16<MSD_DTYPE_BF16, 8, true, false>(p, stream);
   else
     rc = token_order ? launch_fa16<MSD_DTYPE_F16, 8, true, true>(p, stream) : launch_fa16<MSD_DTYPE_F16, 8, true, false>(p, stream);
   if (rc != MSD_OK) return rc;
-  // pass 2: one workgroup per query block over its exclusive list, resuming from pass 1
+#if !defined(MSD_BSA_TWO_PASS)
+  return MSD_OK;
+#endif
+  // (two launches: pass 2, one workgroup per query block over its exclusive list, resuming from pass 1)
+  p.ex_idx = nullptr; p.ex_cnt = nullptr;
   p.blk_idx = t.ex_idx; p.blk_cnt = t.ex_cnt; p.init_cnt = t.init_cnt;
   if (dtype == MSD_DTYPE_BF16)
     return token_order ? launch_fa<MSD_DTYPE_BF16, 4, 32, 64, true, 1, 0, true, true>(p, stream)
