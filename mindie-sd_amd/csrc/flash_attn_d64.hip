@@ -122,7 +122,7 @@ constexpr int kD64Ahead = 3;                          // K operand groups reques
 
 // GEN as in fa_fwd16_kernel (flash_attn_fwd.hip): 0 dense; 1 per-sequence lengths (p.seq_meta) and / or causal;
 // 2 the same with the packed tile numbering; 3 a boolean mask row shared by all queries of a (batch, head).
-// DPAD (dense only): head dims below 64 (p.head_dim, a multiple of 8) computed as 64: the query operand is zero from
+// DPAD: head dims below 64 (p.head_dim, a multiple of 8) computed as 64: the query operand is zero from
 // the real head_dim on, the lanes that would stage the 16-byte chunks of K and V past it request an offset beyond
 // the buffers' range (the DMA writes zeros for them without touching memory), output columns past it are not stored.
 template <int DT, int GEN = 0, bool DPAD = false>
@@ -145,7 +145,6 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
   const int g = lane >> 4;
 
   constexpr bool gen = GEN != 0, keymask = GEN == 3;
-  static_assert(!DPAD || !gen, "padded head dims: dense only");
   const int hd = DPAD ? p.head_dim : 64;
   int bn, qt, b, n, Sq, Skv;
   long long q_tok0, k_tok0;  // general mode: first token of the sequence in packed tensors
@@ -507,12 +506,17 @@ bool fa16_d64_supported(const FaParams& p) {
   return (long long)p.Skv * p.k_ss * 2 < 0x7fffff00ll && (long long)p.Skv * p.v_ss * 2 < 0x7fffff00ll;
 }
 
-int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream) {
-  if (!fa16_d64_supported(p) || D <= 0 || D >= 64 || (D & 7)) return MSD_ERR_UNSUPPORTED;
+int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen) {
+  if (!fa16_d64_supported(p) || D <= 0 || D >= 64 || (D & 7) || gen < 0 || gen > 3) return MSD_ERR_UNSUPPORTED;
   FaParams pp = p;
   pp.head_dim = D;
-  return dtype == MSD_DTYPE_BF16 ? launch_d64<MSD_DTYPE_BF16, 0, true>(pp, stream)
-                                 : launch_d64<MSD_DTYPE_F16, 0, true>(pp, stream);
+  const bool bf = dtype == MSD_DTYPE_BF16;
+  switch (gen) {
+    case 1: return bf ? launch_d64<MSD_DTYPE_BF16, 1, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 1, true>(pp, stream);
+    case 2: return bf ? launch_d64<MSD_DTYPE_BF16, 2, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 2, true>(pp, stream);
+    case 3: return bf ? launch_d64<MSD_DTYPE_BF16, 3, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 3, true>(pp, stream);
+    default: return bf ? launch_d64<MSD_DTYPE_BF16, 0, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 0, true>(pp, stream);
+  }
 }
 
 int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen) {

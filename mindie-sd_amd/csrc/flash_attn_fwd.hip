@@ -1550,8 +1550,19 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   // one mask row for all queries, no other option: the key-mask instantiations of the 16x16x32 kernels
   const bool key_mask = mask && m_sq == 0 && !causal && !seq_meta;
   const bool long_rows = Sq >= kGen16MinRows && Skv > kShortKv;
-  if (D == 64 && long_rows && (!mask || key_mask) && fa16_d64_supported(p))
-    return launch_fa16_d64(p, dtype, stream, key_mask ? 3 : 1);
+  if (long_rows && (!mask || key_mask)) {  // head dims up to 128 on the 16x16x32 kernels, padded where need be
+    const int gen = key_mask ? 3 : 1;
+    if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream, gen);
+    if (D < 64 && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream, gen);
+    if (D > 64 && D < 128 && (long long)Skv * k_ss * 2 < 0x7fffff00ll && (long long)Skv * v_ss * 2 < 0x7fffff00ll) {
+      p.head_dim = D;
+      if (dtype == MSD_DTYPE_BF16)
+        return key_mask ? launch_fa16<MSD_DTYPE_BF16, 8, false, false, 3, true>(p, stream)
+                        : launch_fa16<MSD_DTYPE_BF16, 8, false, false, 1, true>(p, stream);
+      return key_mask ? launch_fa16<MSD_DTYPE_F16, 8, false, false, 3, true>(p, stream)
+                      : launch_fa16<MSD_DTYPE_F16, 8, false, false, 1, true>(p, stream);
+    }
+  }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (key_mask && long_rows) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 3>(p, stream);
@@ -1606,9 +1617,16 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
   p.packed_tiles = (int)tiles;
   // long sequences on average: the 8-wave kernels, whose tiles are 256 rows
   const bool long_rows = total_q / B >= kGen16MinRows && total_k / B > kShortKv;
-  if (D == 64 && long_rows && fa16_d64_supported(p)) {
+  if (D <= 64 && long_rows && fa16_d64_supported(p)) {
     p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
-    return launch_fa16_d64(p, dtype, stream, 2);
+    return D == 64 ? launch_fa16_d64(p, dtype, stream, 2) : launch_fa16_d64_padded(p, dtype, D, stream, 2);
+  }
+  if (D > 64 && D < 128 && long_rows && (long long)total_k * k_ss * 2 < 0x7fffff00ll &&
+      (long long)total_k * v_ss * 2 < 0x7fffff00ll) {
+    p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
+    p.head_dim = D;
+    if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 2, true>(p, stream);
+    return launch_fa16<MSD_DTYPE_F16, 8, false, false, 2, true>(p, stream);
   }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (long_rows) {

@@ -93,11 +93,11 @@ def test_causal_bottom_right(cuda, sq, skv):
     assert torch.isinf(lse.cpu()[:, :, ~seen]).all()
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 96, 40])
 @pytest.mark.parametrize("sq,skv", [(1100, 1100), (1300, 1800), (1800, 1300), (2049, 2049)])
-def test_causal_long_sequences_both_head_dims(cuda, sq, skv, d):
-    """The causal instantiations of the two 16x16x32 kernels (head_dim 128 and 64), three heads (heavy and light
-    tiles are dealt to the XCDs in pairs: an odd and an even tile count)."""
+def test_causal_long_sequences_head_dims(cuda, sq, skv, d):
+    """The causal instantiations of the two 16x16x32 kernels (head_dim 128 and 64; 96 and 40 run padded on them), three
+    heads (heavy and light tiles are dealt to the XCDs in pairs: an odd and an even tile count)."""
     from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
     q, k, v = _rand((2, 3, sq, d), 8), _rand((2, 3, skv, d), 9), _rand((2, 3, skv, d), 10)
     out, lse = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BNSD", return_lse=True, causal=True)
@@ -109,7 +109,8 @@ def test_causal_long_sequences_both_head_dims(cuda, sq, skv, d):
     assert not out.cpu()[:, :, ~seen].any()
     s = (q.float() @ k.float().transpose(-1, -2)) * d ** -0.5
     want_lse = torch.logsumexp(s.masked_fill(~keep, float("-inf")), dim=-1)
-    assert torch.allclose(lse.cpu()[:, :, seen], want_lse[:, :, seen], atol=5e-3, rtol=0)
+    # (the kernel rounds q * scale * log2(e) to 16 bits: 2^-9 of a score that a row with few keys consists of)
+    assert torch.allclose(lse.cpu()[:, :, seen], want_lse[:, :, seen], atol=1e-2, rtol=0)
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -169,7 +170,7 @@ def test_varlen_many_sequences_device_table(cuda, d, causal):
     _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 96, 40])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_varlen_long_sequences(cuda, causal, dtype, d):
@@ -202,7 +203,7 @@ def test_varlen_long_sequences(cuda, causal, dtype, d):
     _check(out_dev, attention_varlen(q2, k2, v2, cq2.tolist(), ck2.tolist(), causal=causal))
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 96, 40])
 @pytest.mark.parametrize("causal", [False, True])
 def test_varlen_many_long_sequences_device_table(cuda, d, causal):
     """70 sequences (more than one wave's worth of table entries) of 1024 tokens and more on average, two of them
@@ -273,7 +274,7 @@ def test_key_padding_mask_expanded_over_queries(cuda):
     _check(out, ref)
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 96, 40])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("per_head", [False, True])
 def test_key_padding_mask_long_sequences(cuda, per_head, dtype, d):
