@@ -74,6 +74,63 @@ def test_masked_or_causal_random_shape(cuda, seed):
     assert err[dense_rows].max().item() <= 2e-2 if dense_rows.any() else True
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_long_random_shape(cuda, seed):
+    """1024 query rows and more, where dense, causal, key-mask and packed calls run on the 16x16x32 kernels at every
+    head_dim (padded where it is not 64, 128 or 256): random lengths off the tile sizes, head dims of every kernel,
+    grouped-query heads, both dtypes."""
+    import mindiesd
+    from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
+    from oracle.attention import attention_varlen
+    r = random.Random(300 + seed)
+    d = r.choice([40, 64, 72, 96, 128, 128, 160, 256])
+    mode = r.choice(["dense", "causal", "keymask", "varlen", "varlen_causal"])
+    sq, skv = r.randrange(1024, 2400), r.randrange(385, 2600)
+    (n, nkv), b = _heads(r), r.choice([1, 2])
+    dtype = r.choice([torch.bfloat16, torch.float16])
+    info = (mode, b, n, nkv, sq, skv, d, dtype)
+    if mode.startswith("varlen"):
+        nseq = r.choice([2, 3, 5])
+        lens_q = [r.choice([0, 1, 200, 1024, 1300, r.randrange(1, 2000)]) for _ in range(nseq)]
+        lens_q[r.randrange(nseq)] = r.randrange(1024, 2200)            # at least one long sequence
+        lens_k = [max(1, l + r.choice([-100, 0, 0, 300])) for l in lens_q]
+        cu_q = torch.tensor([0] + lens_q).cumsum(0).to(torch.int32)
+        cu_k = torch.tensor([0] + lens_k).cumsum(0).to(torch.int32)
+        q, k, v = (_rnd((sum(lens_q), n, d), seed, dtype), _rnd((sum(lens_k), nkv, d), seed + 1, dtype),
+                   _rnd((sum(lens_k), nkv, d), seed + 2, dtype) * 0.5)
+        causal = mode == "varlen_causal"
+        table = (cu_q.to(cuda), cu_k.to(cuda)) if r.random() < 0.5 else (cu_q.tolist(), cu_k.tolist())
+        out = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), *table, causal=causal).cpu()
+        ref = attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal)
+        assert not torch.isnan(out.float()).any()
+        err = (out.float() - ref.float()).abs()
+        assert bool((err <= 5e-2 * ref.float().abs().clamp(min=1.0)).all()), (err.max().item(), info, lens_q, lens_k)
+        return
+    q, k, v = _rnd((b, n, sq, d), seed, dtype), _rnd((b, nkv, skv, d), seed + 1, dtype), _rnd((b, nkv, skv, d), seed + 2, dtype)
+    mask, keep = None, None
+    if mode == "causal":
+        keep = causal_keep_mask(sq, skv)[None, None].expand(b, n, sq, skv)
+    elif mode == "keymask":
+        g = torch.Generator().manual_seed(seed)
+        mask = torch.rand((b, r.choice([1, n]), 1, skv), generator=g) > r.choice([0.1, 0.5, 0.97])
+        if r.random() < 0.5:
+            mask[..., :r.randrange(1, skv)] = False                    # the first tiles hidden
+        keep = mask.expand(b, n, sq, skv)
+    ref = attention_math(q, k.repeat_interleave(n // nkv, 1), v.repeat_interleave(n // nkv, 1), keep, d ** -0.5, head_first=True)
+    if keep is not None:
+        ref = torch.where(keep.any(-1)[..., None], ref, torch.zeros((), dtype=ref.dtype))
+    out = flash_attention(q.to(cuda), k.to(cuda), v.to(cuda), d ** -0.5, "BNSD",
+                          attn_mask=None if mask is None else mask.to(cuda), causal=mode == "causal").cpu()
+    assert not torch.isnan(out.float()).any()
+    err = (out.float() - ref.float()).abs()
+    assert bool((err <= 5e-2 * ref.float().abs().clamp(min=1.0)).all()), (err.max().item(), info)
+    if keep is None:
+        assert err.max().item() <= 2e-2, (err.max().item(), info)
+    else:
+        dense_rows = keep.sum(-1) >= 32
+        assert err[dense_rows].max().item() <= 2e-2 if dense_rows.any() else True, info
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_block_sparse_random_mask(cuda, seed):
     from mindiesd.layers.flash_attn import rainfusion as rf
