@@ -187,9 +187,9 @@ int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen = 
 // head dims below 64 (multiples of 8), computed as 64
 int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen = 0);
 
-// Dense attention at head dims above 128 up to 256 (flash_attn_d256.hip; multiples of 8, computed as 256): no mask,
-// no packed sequences; `supported` as above.
+// Attention at head dims above 128 up to 256 (flash_attn_d256.hip; multiples of 8, computed as 256); `gen` as for
+// launch_fa16_d64 (its packed tiles are 128 rows); `supported` as above.
 bool fa16_d256_supported(const FaParams& p);
-int launch_fa16_d256(const FaParams& p, int dtype, int D, hipStream_t stream);
+int launch_fa16_d256(const FaParams& p, int dtype, int D, hipStream_t stream, int gen = 0);
 
 }  // namespace msd

@@ -1,5 +1,5 @@
-// Dense flash-attention forward for gfx950 (MI355X) at head dims above 128, up to 256: bf16/fp16, no mask, one
-// sequence per batch entry.
+// Flash-attention forward for gfx950 (MI355X) at head dims above 128, up to 256: bf16/fp16; dense, and (from 1024
+// query rows on) causal, packed variable-length sequences and key-padding masks.
 //
 // The reference's fused dense ops (mindiesd/layers/flash_attn/prompt_flash_attn.py:48, fused_attn_score.py:48,
 // csrc/plugin/la.cpp:27-58) take whatever head_dim the model has; the general kernel of flash_attn_hd.hip covers these
@@ -54,7 +54,9 @@ constexpr int kD256Lds = 4 * kD256TileBytes;              // two K and two V sta
 #endif
 constexpr int kD256Ahead = FA16_D256_AHEAD;               // K operand groups requested ahead of their use
 
-template <int DT, bool DPAD>
+// GEN as in fa_fwd16_kernel (flash_attn_fwd.hip): 0 dense; 1 per-sequence lengths (p.seq_meta) and / or causal;
+// 2 the same with the packed tile numbering (128-row tiles here); 3 a boolean mask row shared by all queries.
+template <int DT, bool DPAD, int GEN = 0>
 __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using namespace d256;
@@ -73,17 +75,18 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
   const int c = lane & 15;
   const int g = lane >> 4;
 
+  constexpr bool gen = GEN != 0, keymask = GEN == 3;
   int bn, qt, b, n, Sq, Skv;
-  long long q_tok0, k_tok0;
-  if (!fa16_find_work<0, false>(p, kBM, bn, qt, b, n, Sq, Skv, q_tok0, k_tok0)) return;
+  long long q_tok0, k_tok0;  // general mode: first token of the sequence in packed tensors
+  if (!fa16_find_work<GEN, false>(p, kBM, bn, qt, b, n, Sq, Skv, q_tok0, k_tok0)) return;
   const int nkv = n / (p.N / p.Nkv);
   const int row0 = qt * kBM + wave * 16;  // first query row of this wave
   const int hd = DPAD ? p.head_dim : 256;
 
-  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn;
-  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn;
-  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn;
-  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn;
+  const T* qg = (const T*)p.q + b * p.q_sb + n * p.q_sn + q_tok0 * p.q_ss;
+  const T* kg = (const T*)p.k + b * p.k_sb + nkv * p.k_sn + k_tok0 * p.k_ss;
+  const T* vg = (const T*)p.v + b * p.v_sb + nkv * p.v_sn + k_tok0 * p.v_ss;
+  T* og = (T*)p.o + b * p.o_sb + n * p.o_sn + q_tok0 * p.o_ss;
 
   // ---- Q^T operand, resident: lane (c, g) holds query c, head_dim 32*ks + 8*g .. +8 --------------------------
   X8 qf[8];
@@ -118,10 +121,11 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
   // One instruction moves 2 rows of 512 bytes; a wave issues four per operand and tile (rows 2*wave.. and 16, 32, 48
   // below: the same swizzles, so one per-lane offset per operand serves all four).  Keys past the end of the
   // sequence lie outside the descriptors' range and read as zeros.
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kg, 0, (int)(((long long)(Skv - 1) * p.k_ss + hd) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vg, 0, (int)(((long long)(Skv - 1) * p.v_ss + hd) * 2), 0x00020000);
+  // (a sequence without keys exposes nothing: every row reads as zeros and no tile is computed)
+  const int k_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.k_ss + hd) * 2);
+  const int v_range = gen && Skv <= 0 ? 0 : (int)(((long long)(Skv - 1) * p.v_ss + hd) * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kg, 0, k_range, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vg, 0, v_range, 0x00020000);
   const int k_row_bytes = (int)p.k_ss * 2, v_row_bytes = (int)p.v_ss * 2;
   int k_voff, v_voff;
   {
@@ -163,15 +167,53 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
       v_lds[db] = (unsigned)(uintptr_t)smem + 2 * kTileBytes + key * kRowBytes + ((db ^ (key & 7)) << 5) + 8 * (c & 3);
   }
 
-  const int tiles = (Skv + BN - 1) / BN;
+  // causal: query i sees keys <= i + causal_shift; the last row of this workgroup bounds the tiles it walks
+  const int causal_shift = Skv - Sq;
+  const bool causal = gen && !keymask && p.causal;  // (with a key mask: neither causal nor per-sequence lengths)
+  const int kv_lim = causal ? max(0, min(Skv, qt * kBM + kBM + causal_shift)) : Skv;
+  const int tiles = (kv_lim + BN - 1) / BN;
   load_tile(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   bool first = true;
 
+  // ---- key mask (GEN 3): words of visible keys of the current 64-key tile; bit l of word j = key 4 * l + j (l < 16) --
+  // (see fa_fwd16_kernel: the bytes of the next tile are fetched during the second product and reduced to scalar words)
+  unsigned kvis[4] = {0xffffu, 0xffffu, 0xffffu, 0xffffu};
+  unsigned kraw = 0;  // the lane's four mask bytes of the tile that comes next (lanes 0 .. 15)
+  const unsigned char* mask_g = nullptr;
+  if constexpr (keymask) mask_g = p.mask + b * p.m_sb + n * p.m_sn;
+  auto mask_request = [&](int key0) __attribute__((always_inline)) {  // the load only
+    if constexpr (keymask) {
+      kraw = 0;
+      const int k4 = key0 + 4 * (lane & 15);
+      if (key0 + BN <= Skv) {
+        __builtin_memcpy(&kraw, mask_g + k4, 4);  // (any alignment)
+      } else {                                    // the tile that runs past the row: byte by byte, inside the row
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned byte = mask_g[min(k4 + j, Skv - 1)];
+          kraw |= (k4 + j < Skv ? byte : 0u) << (8 * j);
+        }
+      }
+    }
+  };
+  auto mask_reduce = [&]() __attribute__((always_inline)) {  // bytes -> words in scalar registers
+    if constexpr (keymask) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        kvis[j] = (unsigned)__builtin_amdgcn_ballot_w64(lane < 16 && ((kraw >> (8 * j)) & 0xffu) != 0);
+    }
+  };
+  if constexpr (keymask) {
+    if (tiles > 0) mask_request(0);
+    mask_reduce();
+  }
+
   auto tile_step = [&](auto stage_c, const int key0, const int next_key0) {
     constexpr int stage = decltype(stage_c)::value;
     if (next_key0 >= 0) load_tile(next_key0, stage ^ 1);
+    const unsigned kv_all = kvis[0] & kvis[1] & kvis[2] & kvis[3];
 
     // ---- S^T = K Q^T: 4 accumulation chains of eight; operand reads in groups of 2 key blocks of one 32-wide
     // head_dim step, kAhead groups ahead of the matrix instructions that use them (ring of kAhead + 1) ----------
@@ -213,15 +255,42 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
           if (key0 + 16 * kb + 4 * g + i >= Skv) sacc[kb][i] = -INFINITY;
     }
 
+    // ---- causal: keys beyond the diagonal (the tiles that cross it for some row of this wave) ------------------
+    if constexpr (gen) {
+      if (causal && key0 + BN - 1 > row0 + causal_shift) {
+        const int lim = row0 + c + causal_shift - key0 - 4 * g;  // visible: 16 * kb + i <= lim
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (16 * kb + i > lim) sacc[kb][i] = -INFINITY;
+      }
+    }
+
+    // ---- key mask: tiles that hide some of their keys ----------------------------------------------------------
+    if constexpr (keymask) {
+      if (kv_all != 0xffffu) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned w = kvis[i] >> g;  // key 16 * kb + 4 * g + i is bit 4 * kb + g of word i
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb)
+            if (!((w >> (4 * kb)) & 1u)) sacc[kb][i] = -INFINITY;
+        }
+      }
+    }
+
     // ---- online softmax (exp2 domain): the reference maximum moves only when some row of the wave exceeds it by
     // more than 2^kTau (or on the first tile), so most tiles rescale nothing -------------------------------------
     X8 pf[2];
+    bool seen = !keymask;  // key mask: this tile showed some row of the wave a key (all rows share the mask)
     {
       float mx = sacc[0][0];
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sacc[kb][i]);
+      if constexpr (keymask) seen = __builtin_amdgcn_ballot_w64(mx > -INFINITY) != 0;
       // (the test needs no row maximum: some lane's part exceeds the threshold iff some row's maximum does)
       l_run += lt[0];
       if (first || __builtin_amdgcn_ballot_w64(mx > kTau) != 0) {
@@ -268,6 +337,9 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
         dst[2 * d4 + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(v_lds[db & 7]);
       });
     };
+    if constexpr (keymask) {
+      if (next_key0 >= 0) mask_request(next_key0);  // lands during the second product
+    }
     issue(std::integral_constant<int, 0>{}, vf[0]);
     static_for<8>([&](auto step_c) __attribute__((always_inline)) {
       constexpr int s = decltype(step_c)::value;
@@ -289,8 +361,9 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
         lt = E::mfma16(ones, pf[j], j == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : lt);
     });
 
-    first = false;
+    first = first && !seen;  // (without a key mask: false from the first tile on)
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the next tile has landed
+    mask_reduce();
     __syncthreads();
   };
   for (int t = 0; t < tiles; t += 2) {
@@ -332,12 +405,12 @@ __global__ __launch_bounds__(kD256Waves * 64, 1) void fa_fwd16_d256_kernel(const
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int DT, bool DPAD>
+template <int DT, bool DPAD, int GEN>
 static int launch_d256(const FaParams& p, hipStream_t stream) {
-  auto kern = fa_fwd16_d256_kernel<DT, DPAD>;
+  auto kern = fa_fwd16_d256_kernel<DT, DPAD, GEN>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kD256Lds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const long long grid = fa16_grid<0, false>(p, kD256Waves * 16);
+  const long long grid = fa16_grid<GEN, false>(p, kD256Waves * 16);
   if (grid > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kD256Waves * 64), kD256Lds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
@@ -349,13 +422,24 @@ bool fa16_d256_supported(const FaParams& p) {
   return (long long)p.Skv * p.k_ss * 2 < 0x7fffff00ll && (long long)p.Skv * p.v_ss * 2 < 0x7fffff00ll;
 }
 
-int launch_fa16_d256(const FaParams& p, int dtype, int D, hipStream_t stream) {
-  if (!fa16_d256_supported(p) || D <= 128 || D > 256 || (D & 7)) return MSD_ERR_UNSUPPORTED;
+template <int DT, bool DPAD>
+static int launch_d256_gen(const FaParams& p, int gen, hipStream_t stream) {
+  switch (gen) {
+    case 1: return launch_d256<DT, DPAD, 1>(p, stream);
+    case 2: return launch_d256<DT, DPAD, 2>(p, stream);
+    case 3: return launch_d256<DT, DPAD, 3>(p, stream);
+    default: return launch_d256<DT, DPAD, 0>(p, stream);
+  }
+}
+
+int launch_fa16_d256(const FaParams& p, int dtype, int D, hipStream_t stream, int gen) {
+  if (!fa16_d256_supported(p) || D <= 128 || D > 256 || (D & 7) || gen < 0 || gen > 3) return MSD_ERR_UNSUPPORTED;
   const bool bf = dtype == MSD_DTYPE_BF16;
-  if (D == 256) return bf ? launch_d256<MSD_DTYPE_BF16, false>(p, stream) : launch_d256<MSD_DTYPE_F16, false>(p, stream);
+  if (D == 256)
+    return bf ? launch_d256_gen<MSD_DTYPE_BF16, false>(p, gen, stream) : launch_d256_gen<MSD_DTYPE_F16, false>(p, gen, stream);
   FaParams pp = p;
   pp.head_dim = D;
-  return bf ? launch_d256<MSD_DTYPE_BF16, true>(pp, stream) : launch_d256<MSD_DTYPE_F16, true>(pp, stream);
+  return bf ? launch_d256_gen<MSD_DTYPE_BF16, true>(pp, gen, stream) : launch_d256_gen<MSD_DTYPE_F16, true>(pp, gen, stream);
 }
 
 }  // namespace msd

@@ -1562,6 +1562,7 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
       return key_mask ? launch_fa16<MSD_DTYPE_F16, 8, false, false, 3, true>(p, stream)
                       : launch_fa16<MSD_DTYPE_F16, 8, false, false, 1, true>(p, stream);
     }
+    if (D > 128 && fa16_d256_supported(p)) return launch_fa16_d256(p, dtype, D, stream, gen);
   }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (key_mask && long_rows) {
@@ -1627,6 +1628,10 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
     p.head_dim = D;
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 2, true>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 2, true>(p, stream);
+  }
+  if (D > 128 && long_rows && (long long)total_k * k_ss * 2 < 0x7fffff00ll && (long long)total_k * v_ss * 2 < 0x7fffff00ll) {
+    p.packed_tiles = (int)(((long long)total_q + 127) / 128 + B);  // (this kernel's tiles are 128 rows)
+    return launch_fa16_d256(p, dtype, D, stream, 2);
   }
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   if (long_rows) {
