@@ -1,4 +1,4 @@
-// Flash-attention forward for gfx950 (MI355X) at head dims above 128, up to 256: bf16/fp16; dense, and (from 1024
+// Flash-attention forward for gfx950 (MI355X) at head dims above 128, up to 256: bf16/fp16; dense, and (from 256
 // query rows on) causal, packed variable-length sequences and key-padding masks.
 //
 // The reference's fused dense ops (mindiesd/layers/flash_attn/prompt_flash_attn.py:48, fused_attn_score.py:48,

@@ -1,4 +1,4 @@
-// Flash-attention forward for gfx950 (MI355X) at head_dim 64: bf16/fp16; dense, and (from 1024 query rows on) causal,
+// Flash-attention forward for gfx950 (MI355X) at head_dim 64: bf16/fp16; dense, and (from 256 query rows on) causal,
 // packed variable-length sequences and key-padding masks.
 //
 // head_dim 64 is what the reference's own tests of attention_forward run

@@ -7,7 +7,7 @@
 // csrc/plugin/rainfusionattention.cpp:27-64).
 //
 // Two kernels share the algorithm: fa_fwd16_kernel (16x16x32 matrix instruction: plain dense attention, and causal
-// and packed variable-length attention without a boolean mask from 1024 query rows on) and fa_fwd_kernel (32x32x16
+// and packed variable-length attention without a boolean mask from 256 query rows on) and fa_fwd_kernel (32x32x16
 // instruction: block-sparse and masked attention, the short causal / variable-length cases and the tuning variants
 // of the dense case).  What follows describes fa_fwd_kernel; fa_fwd16_kernel states its differences.
 //
@@ -1310,7 +1310,10 @@ extern "C" {
 
 constexpr int kShortKv = 384;  // dense calls with at most this many keys run on the 4-wave kernel (see below)
 // general mode: query rows (of the longest sequence; packed: of the average one) from which the 8-wave kernel is used
-constexpr int kGen16MinRows = 1024;
+#ifndef MSD_GEN16_MIN_ROWS
+#define MSD_GEN16_MIN_ROWS 256
+#endif
+constexpr int kGen16MinRows = MSD_GEN16_MIN_ROWS;
 
 static int check_common(const void* q, const void* k, const void* v, const void* out, int dtype, int B, int N,
                         int Nkv, int Sq, int Skv, int D, const long long* st, float scale, bool any_head_dim = false) {

@@ -73,7 +73,7 @@ def test_mask_dtypes_and_fully_masked_rows(cuda):
     assert torch.equal(out[:, :, rows], v[:, :, 17:18].expand(1, 2, 129, 128))  # one visible key: the output is its value row
 
 
-# (from 1024 query rows on, calls without a mask run on the 8-wave kernel's general instantiation)
+# (from 256 query rows on, calls without a mask run on the 8-wave kernel's general instantiation)
 @pytest.mark.parametrize("sq,skv", [(256, 256), (300, 300), (77, 500), (500, 77), (1000, 1300), (1100, 1100),
                                     (1300, 1800), (1800, 1300), (1025, 2047), (1536, 385)])
 def test_causal_bottom_right(cuda, sq, skv):
@@ -174,7 +174,7 @@ def test_varlen_many_sequences_device_table(cuda, d, causal):
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_varlen_long_sequences(cuda, causal, dtype, d):
-    """Sequences of 1024 query tokens and more take the 8-wave kernel (256-row tiles): lengths around the tile edges,
+    """Long sequences on the 8-wave kernel (256-row tiles): lengths around the tile edges,
     key counts above and below the query counts (causal rows without any visible key give zeros), a sequence without
     keys and one without queries, grouped heads.  Host lists size the grid by the longest sequence; device tables
     of long sequences number the tiles through the table."""
@@ -280,7 +280,7 @@ def test_key_padding_mask_expanded_over_queries(cuda):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("per_head", [False, True])
 def test_key_padding_mask_long_sequences(cuda, per_head, dtype, d):
-    """From 1024 query rows on, a mask row shared by all queries runs on the 8-wave kernel (mask bytes reduced to
+    """From 256 query rows on, a mask row shared by all queries runs on the 8-wave kernel (mask bytes reduced to
     words of visible keys per tile).  Trailing padding, holes, a random half, a row that hides its first two key tiles,
     a batch entry without any visible key (zeros); key count off the tile size, mask rows at odd addresses."""
     import mindiesd

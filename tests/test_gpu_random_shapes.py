@@ -76,7 +76,7 @@ def test_masked_or_causal_random_shape(cuda, seed):
 
 @pytest.mark.parametrize("seed", range(40))
 def test_long_random_shape(cuda, seed):
-    """1024 query rows and more, where dense, causal, key-mask and packed calls run on the 16x16x32 kernels at every
+    """Long sequences, where dense, causal, key-mask and packed calls run on the 16x16x32 kernels at every
     head_dim (padded where it is not 64, 128 or 256): random lengths off the tile sizes, head dims of every kernel,
     grouped-query heads, both dtypes."""
     import mindiesd
