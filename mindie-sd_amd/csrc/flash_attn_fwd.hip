@@ -1308,7 +1308,10 @@ using namespace msd;
 
 extern "C" {
 
-constexpr int kShortKv = 384;  // dense calls with at most this many keys run on the 4-wave kernel (see below)
+#ifndef MSD_SHORT_KV
+#define MSD_SHORT_KV 384
+#endif
+constexpr int kShortKv = MSD_SHORT_KV;  // dense calls with at most this many keys run on the 4-wave kernel (see below)
 // general mode: query rows (of the longest sequence; packed: of the average one) from which the 8-wave kernel is used
 #ifndef MSD_GEN16_MIN_ROWS
 #define MSD_GEN16_MIN_ROWS 256
@@ -1461,14 +1464,16 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   // Head dims between 64 and 128 run as head_dim 128 on the 16x16x32 kernel (the part of the matrix work spent on
   // the padding costs less than the general kernel's staging through registers: 72 -> 580 vs 730 TFLOP/s of real
   // work, 112 -> 800 vs 1130), when the 256-byte rows the DMA fetches stay inside the kernel's 32-bit offsets.
-  if (D > 64 && D < 128 && Skv > kShortKv && (long long)Skv * k_ss * 2 < 0x7fffff00ll &&
+  if (D > 64 && D < 128 && (long long)Skv * k_ss * 2 < 0x7fffff00ll &&
       (long long)Skv * v_ss * 2 < 0x7fffff00ll) {  // (below the offset that stands for "no data" in the kernel)
     p.head_dim = D;
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 0, true>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 0, true>(p, stream);
   }
-  if (D > 128 && Skv > kShortKv && fa16_d256_supported(p)) return launch_fa16_d256(p, dtype, D, stream);
-  if (D < 64 && Skv > kShortKv && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream);
+  // (the rule for short key sequences below is head_dim 128's alone: at the other widths the alternative is the
+  // general kernel, which these beat at 77 keys already)
+  if (D > 128 && fa16_d256_supported(p)) return launch_fa16_d256(p, dtype, D, stream);
+  if (D < 64 && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream);
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   // A few key tiles per query tile (cross attention over a short text): the launch is mostly reading Q and writing O,
   // and two 4-wave workgroups per CU overlap one's memory phases with the other's tiles better than one 8-wave
@@ -1552,7 +1557,7 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
   p.mask = mask; p.m_sb = m_sb; p.m_sn = m_sn; p.m_sq = m_sq;
   // one mask row for all queries, no other option: the key-mask instantiations of the 16x16x32 kernels
   const bool key_mask = mask && m_sq == 0 && !causal && !seq_meta;
-  const bool long_rows = Sq >= kGen16MinRows && Skv > kShortKv;
+  const bool long_rows = Sq >= kGen16MinRows && (D != 128 || Skv > kShortKv);
   if (long_rows && (!mask || key_mask)) {  // head dims up to 128 on the 16x16x32 kernels, padded where need be
     const int gen = key_mask ? 3 : 1;
     if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream, gen);
@@ -1620,7 +1625,7 @@ int mindiesd_flash_attention_packed_fwd(const void* q, const void* k, const void
   if (tiles * N > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
   p.packed_tiles = (int)tiles;
   // long sequences on average: the 8-wave kernels, whose tiles are 256 rows
-  const bool long_rows = total_q / B >= kGen16MinRows && total_k / B > kShortKv;
+  const bool long_rows = total_q / B >= kGen16MinRows && (D != 128 || total_k / B > kShortKv);
   if (D <= 64 && long_rows && fa16_d64_supported(p)) {
     p.packed_tiles = (int)(((long long)total_q + 255) / 256 + B);
     return D == 64 ? launch_fa16_d64(p, dtype, stream, 2) : launch_fa16_d64_padded(p, dtype, D, stream, 2);

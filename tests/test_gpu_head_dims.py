@@ -108,7 +108,10 @@ def test_varlen(cuda, d, causal):
     _check(out, ref)
     cu_q_d, cu_k_d = (torch.tensor(c, dtype=torch.int32, device=cuda) for c in (cu_q, cu_k))
     out2 = mindiesd.attention_forward_varlen(q.to(cuda), k.to(cuda), v.to(cuda), cu_q_d, cu_k_d, causal=causal).cpu()
-    assert torch.equal(out, out2)
+    # (host lists size the launch by the longest sequence, device tables by the average: the two may take different
+    # kernels, equal up to the summation order)
+    assert (out.float() - out2.float()).abs().max() <= 2.0 ** -7
+    _check(out2, ref)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

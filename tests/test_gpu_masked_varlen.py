@@ -166,7 +166,9 @@ def test_varlen_many_sequences_device_table(cuda, d, causal):
     dev = [t.to(cuda) for t in (q, k, v)]
     out_dev = mindiesd.attention_forward_varlen(*dev, cu_q.to(cuda), cu_k.to(cuda), causal=causal).cpu()
     out_host = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
-    assert torch.equal(out_dev, out_host)
+    # (host lists size the launch by the longest sequence, device tables by the average: the two may take different
+    # kernels, equal up to the summation order)
+    assert (out_dev.float() - out_host.float()).abs().max() <= 2.0 ** -6
     _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
 
 
@@ -201,7 +203,9 @@ def test_varlen_long_sequences(cuda, causal, dtype, d):
     dev2 = [t.to(cuda) for t in (q2, k2, v2)]
     out_dev = mindiesd.attention_forward_varlen(*dev2, cq2.to(cuda), ck2.to(cuda), causal=causal).cpu()
     out_host = mindiesd.attention_forward_varlen(*dev2, cq2.tolist(), ck2.tolist(), causal=causal).cpu()
-    assert torch.equal(out_dev, out_host)
+    # (host lists size the launch by the longest sequence, device tables by the average: the two may take different
+    # kernels, equal up to the summation order)
+    assert (out_dev.float() - out_host.float()).abs().max() <= 2.0 ** -6
     _check(out_dev, attention_varlen(q2, k2, v2, cq2.tolist(), ck2.tolist(), causal=causal))
 
 
@@ -226,7 +230,9 @@ def test_varlen_many_long_sequences_device_table(cuda, d, causal):
     dev = [t.to(cuda) for t in (q, k, v)]
     out_dev = mindiesd.attention_forward_varlen(*dev, cu_q.to(cuda), cu_k.to(cuda), causal=causal).cpu()
     out_host = mindiesd.attention_forward_varlen(*dev, cu_q.tolist(), cu_k.tolist(), causal=causal).cpu()
-    assert torch.equal(out_dev, out_host)
+    # (host lists size the launch by the longest sequence, device tables by the average: the two may take different
+    # kernels, equal up to the summation order)
+    assert (out_dev.float() - out_host.float()).abs().max() <= 2.0 ** -6
     _check(out_dev, attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), causal=causal))
 
 
