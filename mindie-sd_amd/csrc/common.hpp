@@ -251,7 +251,7 @@ __device__ __forceinline__ void cond_rescale_fa16(int flag, float delta, float a
   o7 = f32x4_t{o7_0, o7_1, o7_2, o7_3};
 }
 
-// Pair tables of the two-pass block-sparse attention (built by bsa_pair.hip, consumed by flash_attn_fwd.hip).
+// Pair tables of the block-sparse attention over paired query blocks (built by bsa_pair.hip, consumed by flash_attn_fwd.hip).
 struct BsaPairTables {
   int* pairs;     // [BN][NP][2]
   int* sh_idx;    // [BN][NP][KB]

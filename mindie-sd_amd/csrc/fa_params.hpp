@@ -27,7 +27,7 @@ struct FaParams {
   int QB;
   const int* order;  // optional [B*N*QB] work order (heaviest query blocks first)
   const int* tok;    // GATHER instantiations: [Sq] row of q/out that holds the token at query position i
-  // two-pass block-sparse attention over paired query blocks (see bsa_pair.hip)
+  // block-sparse attention over paired query blocks (see bsa_pair.hip)
   const int* pairs;     // PAIR kernel: [B * N][NP][2] query blocks of a pair (second -1: none); lists are per pair
   int NP;
   float* state;         // [B * N][Sq] log2-domain log-sum-exp after the first pass (written by it, read by the second)

@@ -1391,11 +1391,10 @@ int mindiesd_block_sparse_attention_gather_fwd(const void* q, const void* k, con
   return launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, true>(p, stream);
 }
 
-// Block-sparse attention driven by the int8 mask itself, in two passes over paired query blocks (bsa_pair.hip):
-// pairing + lists, then the key blocks both partners of a pair selected (256-row workgroups, the dense kernel's
-// inner loop), then what only one of them selected, continuing the running softmax.  Same result as
-// mindiesd_block_sparse_attention_fwd on the lists of the mask up to the order of accumulation and one more
-// rounding to the 16-bit output type: the first pass hands its normalised rows to the second through `out`.
+// Block-sparse attention driven by the int8 mask itself, over paired query blocks (bsa_pair.hip): pairing + lists,
+// then one 256-row workgroup per pair: the key blocks both partners selected (the dense kernel's inner loop), then
+// what only one of them selected, with that partner's four waves, the running softmax going on.  Same result as
+// mindiesd_block_sparse_attention_fwd on the lists of the mask up to the order of accumulation.
 size_t mindiesd_block_sparse_attention_paired_workspace_size(int B, int N, int Sq, int Skv) {
   if (B <= 0 || N <= 0 || Sq <= 0 || Skv <= 0) return 0;
   const long long BN = (long long)B * N;

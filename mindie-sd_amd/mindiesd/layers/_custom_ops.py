@@ -211,7 +211,7 @@ def _rainfusionattention_impl(query, key, value, select_idx, select_num_idx, blo
         raise RuntimeError("select_idx must be [q_blocks, N, kv_blocks] and select_num_idx [q_blocks, N]")
     # The selection as an int8 mask: entry j of a row counts if j < select_num_idx and the id names a key block
     # (ids outside [0, kv_blocks) and entries past the count are dropped, so a malformed list cannot make the
-    # kernel read outside its tables).  The mask form runs the paired two-pass kernel.
+    # kernel read outside its tables).  The mask form runs the kernel over paired query blocks.
     skv = max(lens_kv) if unequal else (k4.shape[2] if layout == "BNSD" else k4.shape[1])
     kb = (skv + 127) // 128
     sel = select_idx.permute(1, 0, 2).to(torch.int64)                               # [N, qb, width]

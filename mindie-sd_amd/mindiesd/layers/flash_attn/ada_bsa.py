@@ -82,7 +82,7 @@ def ada_block_sparse_attention(query, key, value, sparse_mask, sparse_count_tabl
     if sparse_count_table is not None and tuple(sparse_count_table.shape) != (b, n, nb):
         raise RuntimeError(f"sparse_count_table must be [B, N, {nb}], got {tuple(sparse_count_table.shape)}")
     if not causal and q.shape[-1] == HEAD_DIM:
-        # without the in-block causal test this is plain block-sparse attention: the two-pass kernel over paired
+        # without the in-block causal test this is plain block-sparse attention: the kernel over paired
         # query blocks, driven by the mask itself
         return block_sparse_attention_mask(q, k, v, sparse_mask[..., :nb], scale_value, input_layout)
     idx, cnt = mask_to_lists(sparse_mask)

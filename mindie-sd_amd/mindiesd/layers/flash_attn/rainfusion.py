@@ -371,7 +371,7 @@ def block_sparse_attention_mask(query, key, value, block_sparse_mask, scale, lay
                                 order=None):
     """Attention of every 128-row query block over the key blocks its mask row selects
     (``block_sparse_mask`` int8/bool [B, N, qb, kb], non-zero = attend; an all-zero row yields zeros).
-    Runs the two-pass kernel over paired query blocks (query blocks with similar mask rows share their K/V
+    Runs the kernel over paired query blocks (query blocks with similar mask rows share their K/V
     tiles); masks too large for the pairing kernels go through the block lists.  ``order`` as in
     :func:`block_sparse_attention_lists`."""
     for name, t in (("query", query), ("key", key), ("value", value)):

@@ -1,4 +1,4 @@
-"""GPU parity of the two-pass block-sparse attention over paired query blocks (mindiesd_block_sparse_attention_paired_fwd)
+"""GPU parity of the block-sparse attention over paired query blocks (mindiesd_block_sparse_attention_paired_fwd)
 against the CPU oracle (the reference's numpy model of its block-sparse kernel,
 tests/plugin/test_block_sparse_attention.py:32-65) within the reference's kernel rule |err| <= 2^-6 * max(1, |golden|),
 and against the one-pass list kernel on the same mask."""
