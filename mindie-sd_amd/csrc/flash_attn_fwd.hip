@@ -37,6 +37,13 @@
 
 namespace msd {
 
+// An entry of a device table read through the scalar unit (pointer and index wave-uniform): the value arrives in a
+// scalar register and is waited for where it is first used, not where it is requested - a vector load followed by a
+// readfirstlane stalls the wave for the whole memory latency at the request.
+__device__ __forceinline__ int scalar_load(const int* p, int i) {
+  return ((const __attribute__((address_space(4))) int*)p)[i];
+}
+
 template <int DT, int NWAVES, int QPW, int BN, bool SPARSE>
 struct FaCfg {
   static constexpr int kD = 128;
@@ -830,8 +837,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
     const long long pair_lin = (long long)bn * p.NP + qt;
     l_ptr = p.blk_idx + pair_lin * p.kb_stride;
     l_n = __builtin_amdgcn_readfirstlane(p.blk_cnt[pair_lin]);
-    if (l_n > 0) id_a = __builtin_amdgcn_readfirstlane(l_ptr[0]);
-    if (l_n > 1) id_b = __builtin_amdgcn_readfirstlane(l_ptr[1]);
+    if (l_n > 0) id_a = scalar_load(l_ptr, 0);
+    if (l_n > 1) id_b = scalar_load(l_ptr, 1);
     if (l_n > 0) load_tile(id_a * BN, 0);
   } else {
     load_tile(0, 0);
@@ -1040,8 +1047,8 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
   };
   if constexpr (PAIR) {
     for (int pos = 0; pos < l_n; pos += 2) {
-      const int id_c = __builtin_amdgcn_readfirstlane(l_ptr[pos + 2 < l_n ? pos + 2 : 0]);
-      const int id_d = __builtin_amdgcn_readfirstlane(l_ptr[pos + 3 < l_n ? pos + 3 : 0]);
+      const int id_c = scalar_load(l_ptr, pos + 2 < l_n ? pos + 2 : 0);
+      const int id_d = scalar_load(l_ptr, pos + 3 < l_n ? pos + 3 : 0);
       tile_step(std::integral_constant<int, 0>{}, id_a * BN, pos + 1 < l_n ? id_b * BN : -1);
       if (pos + 1 < l_n) tile_step(std::integral_constant<int, 1>{}, id_b * BN, pos + 2 < l_n ? id_c * BN : -1);
       id_a = id_c;
@@ -1063,21 +1070,17 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
       const int e_o = qb_other >= 0 ? __builtin_amdgcn_readfirstlane(p.ex_cnt[(long long)bn * p.QB + qb_other]) : 0;
       const int my_steps = 2 * e_n, steps = 2 * max(e_n, e_o);
       // this group's halves of the stages; its waves stage rows 4 * w4 + 16 * i of a sub-tile
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) k_lds[ks] += grp * kHalf;
-#pragma unroll
-      for (int db = 0; db < 4; ++db) v_lds[db] += grp * kHalf;
-      k_voff -= 16 * grp * k_row_bytes;
-      v_voff -= 16 * grp * v_row_bytes;
       auto load_half = [&](int key0, int stage) {
         MSD_LDS char* kb = smem + stage * kTileBytes + grp * kHalf;
         MSD_LDS char* vb = smem + (2 + stage) * kTileBytes + grp * kHalf;
+        const int g16 = 16 * grp;
+        const int kvo = k_voff - g16 * k_row_bytes, vvo = v_voff - g16 * v_row_bytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int g4 = i * 4 + w4;  // 4-row group of the sub-tile
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g4 * 1024), 16, k_voff,
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (MSD_LDS void*)(kb + g4 * 1024), 16, kvo,
                                                    (key0 + 16 * i) * k_row_bytes, 0, 0);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g4 * 1024), 16, v_voff,
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (MSD_LDS void*)(vb + g4 * 1024), 16, vvo,
                                                    (key0 + 16 * i) * v_row_bytes, 0, 0);
         }
       };
@@ -1085,7 +1088,10 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
         constexpr int stage = decltype(stage_c)::value;
         if (next_key0 >= 0) load_half(next_key0, stage ^ 1);
         if (key0 >= 0) {
-          // S^T = K Q^T over 4 key blocks (see tile_step)
+          // S^T = K Q^T over 4 key blocks (see tile_step), read from this group's half of the stage
+          unsigned kl[4];
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) kl[ks] = k_lds[ks] + grp * kHalf;
           f32x4_t sacc[4][2];
           constexpr int kAhead = FA16_AHEAD;
           X8 afrag[kAhead + 1][2];
@@ -1094,7 +1100,7 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
             constexpr int ks = gi >> 1, qu = gi & 1;
 #pragma unroll
             for (int i = 0; i < 2; ++i)
-              dst[i] = *(MSD_LDS const X8*)(uintptr_t)(k_lds[ks] + stage * kTileBytes + (2 * qu + i) * 16 * kRowBytes);
+              dst[i] = *(MSD_LDS const X8*)(uintptr_t)(kl[ks] + stage * kTileBytes + (2 * qu + i) * 16 * kRowBytes);
           };
           static_for<kAhead>([&](auto gi_c) __attribute__((always_inline)) { k_read(gi_c, afrag[decltype(gi_c)::value]); });
           static_for<8>([&](auto gi_c) __attribute__((always_inline)) {
@@ -1165,13 +1171,16 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
             }
           }
           s16x4_t vf[2][8];
+          unsigned vl[4];
+#pragma unroll
+          for (int d4 = 0; d4 < 4; ++d4) vl[d4] = v_lds[d4] + grp * kHalf;
           auto issue = [&](auto step_c, s16x4_t(&dst)[8]) __attribute__((always_inline)) {
             constexpr int s = decltype(step_c)::value;
             constexpr int j = s >> 1, dbh = s & 1;
             constexpr int off = stage * kTileBytes + 32 * j * kRowBytes;
 #pragma unroll
             for (int d4 = 0; d4 < 4; ++d4) {
-              const unsigned a = v_lds[d4] ^ (dbh << 7);
+              const unsigned a = vl[d4] ^ (dbh << 7);
               dst[2 * d4] = lds_read_tr16_async<off>(a);
               dst[2 * d4 + 1] = lds_read_tr16_async<off + 16 * kRowBytes>(a);
             }
@@ -1206,12 +1215,12 @@ __global__ __launch_bounds__(NWAVES * 64, 1) void fa_fwd16_kernel(const FaParams
         __syncthreads();
       };
       // key of sub-tile st of this group (-1: past its list); the block ids come by scalar loads one block ahead
-      int e_cur = my_steps > 0 ? __builtin_amdgcn_readfirstlane(e_ptr[0]) : 0;
+      int e_cur = my_steps > 0 ? scalar_load(e_ptr, 0) : 0;
       if (my_steps > 0) load_half(e_cur * 128, 0);
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
       for (int st = 0; st < steps; st += 2) {  // one 128-key block per iteration: its two halves
-        const int e_next = st + 2 < my_steps ? __builtin_amdgcn_readfirstlane(e_ptr[(st >> 1) + 1]) : 0;
+        const int e_next = st + 2 < my_steps ? scalar_load(e_ptr, (st >> 1) + 1) : 0;
         const bool mine = st < my_steps;
         half_step(std::integral_constant<int, 0>{}, mine ? e_cur * 128 : -1, mine ? e_cur * 128 + 64 : -1);
         half_step(std::integral_constant<int, 1>{}, mine ? e_cur * 128 + 64 : -1, st + 2 < my_steps ? e_next * 128 : -1);
