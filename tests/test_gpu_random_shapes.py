@@ -1,7 +1,7 @@
 """GPU parity on shapes drawn at random (fixed seeds): sequence lengths around every tile and block boundary, unequal
 query / key lengths, grouped-query heads, both layouts and dtypes, head dims of every kernel, random boolean masks,
-causal masks and random block masks, each against the CPU oracle with the tolerance of the path's own test file;
-the two quantisers bit for bit on values spread over many octaves, tiny values, values on a coarse grid (rounding
+causal masks and random block masks, the MXFP8 GEMM with and without SwiGLU and bias, each against the CPU oracle
+with the tolerance of the path's own test file; the two quantisers bit for bit on values spread over many octaves, tiny values, values on a coarse grid (rounding
 ties) and outliers."""
 import random
 
@@ -301,3 +301,30 @@ def test_ada_attention_random_mask(cuda, seed):
     assert not torch.isnan(out.float()).any()
     eb, ok, mx = oa.ref_compare(want, out, 2.0 ** -6)
     assert ok, (eb, mx, b, n, nkv, s, causal, layout, dtype)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_mxfp8_gemm_random_shape(cuda, seed):
+    """MXFP8 GEMM on random shapes: row counts off the 256-row tiles (1 row up), K any multiple of 128, output widths
+    off the tile widths, with and without SwiGLU and bias, both output dtypes; within 2^-7 relative + 1e-3 of the
+    oracle's exact product of the dequantised operands (tests/test_gpu_mxfp8_gemm.py's bound)."""
+    from mindiesd.layers.quant import mx_quantize, mxfp8_matmul
+    from oracle import quant as oq
+    r = random.Random(900 + seed)
+    m = r.choice([1, 7, 255, 256, 257, 511, 513, r.randrange(1, 1500)])
+    k = 128 * r.randrange(1, 13)
+    swiglu = r.random() < 0.5
+    n = (16 if swiglu else 8) * r.randrange(1, 80)
+    out_dtype = r.choice([torch.bfloat16, torch.float16])
+    x, w = _rnd((m, k), seed, torch.bfloat16), _rnd((n, k), seed + 1, torch.bfloat16) * 0.05
+    bias = _rnd((n,), seed + 2, torch.float32) if r.random() < 0.5 else None
+    y = oq.mxfp8_gemm(x, w, bias)
+    if swiglu:
+        gate, up = y[:, :n // 2], y[:, n // 2:]
+        y = gate / (1.0 + torch.exp(-gate)) * up
+    xq, xs = mx_quantize(x.to(cuda))
+    wq, ws = mx_quantize(w.to(cuda))
+    out = mxfp8_matmul(xq, xs, wq, ws, None if bias is None else bias.to(cuda), out_dtype, swiglu=swiglu).cpu()
+    assert out.shape == (m, n // 2 if swiglu else n) and out.dtype == out_dtype
+    err = (out.double() - y).abs()
+    assert bool((err <= 2.0 ** -7 * y.abs() + 1e-3).all()), (err.max().item(), m, k, n, swiglu, bias is not None, out_dtype)
