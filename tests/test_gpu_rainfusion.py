@@ -286,3 +286,9 @@ def test_op_argument_errors(cuda):
         mindiesd.sparse_attention(q, q, q, input_layout="SBH")
     with pytest.raises(mindiesd.ParametersInvalid):
         mindiesd.sparse_attention(q, q, q, sparse_type="topk")
+    # 160 image + 77 text tokens: the pooled parts make 2 + 1 blocks, the sequence has 2 - the mask cannot fit the
+    # attention (rf_v3.py:219 documents text lengths other than 0 as unsupported), so the call is refused
+    from mindiesd.layers.flash_attn.rainfusion import bsa_sparse_attention_v3
+    x = torch.randn(1, 2, 237, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(mindiesd.ParametersInvalid):
+        bsa_sparse_attention_v3(x, x, x, (1, 8, 20), txt_len=77, input_layout="BNSD")
