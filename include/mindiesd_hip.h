@@ -16,9 +16,10 @@
  * pytorch_npu_helper.h:646-649).
  *
  * dtype codes: 0 = bf16, 1 = fp16.  All tensors have head_dim D contiguous in memory: D = 128 everywhere,
- * except that the two dense entry points (mindiesd_flash_attention_fwd, mindiesd_flash_attention_general_fwd)
- * also take every multiple of 8 up to 256 (a generic kernel; the reference's own attention_forward tests run
- * head_dim 64, tests/layers/flash_attn/test_attn_forward.py:31-169).  Pointers must
+ * except that the three dense entry points (mindiesd_flash_attention_fwd, mindiesd_flash_attention_general_fwd,
+ * mindiesd_flash_attention_packed_fwd) also take every multiple of 8 up to 256 (kernels of their own at 64, up to
+ * 128 and up to 256, narrower head dims computed at the next of these widths; the reference's own
+ * attention_forward tests run head_dim 64, tests/layers/flash_attn/test_attn_forward.py:31-169).  Pointers must
  * be 16-byte aligned and every stride a multiple of 8 elements.  "strides" are element strides of the
  * (batch, head, token) dimensions, so BNSD and BSND tensors are both passed without a copy.
  */
