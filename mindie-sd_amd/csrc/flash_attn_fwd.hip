@@ -25,6 +25,7 @@
 // LDS layouts (bank-conflict free for their readers, no padding):
 //     K tile [key][128]: 16-byte chunk c of row key is stored at chunk c ^ (key & 15)
 //     V tile [key][128]: 64-byte chunk c of row key is stored at chunk c ^ (key & 3)
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -1320,6 +1321,7 @@ extern "C" {
 #ifndef MSD_SHORT_KV
 #define MSD_SHORT_KV 384
 #endif
+constexpr int kCus = 256;  // compute units of the MI355X
 constexpr int kShortKv = MSD_SHORT_KV;  // dense calls with at most this many keys run on the 4-wave kernel (see below)
 // general mode: query rows (of the longest sequence; packed: of the average one) from which the 8-wave kernel is used
 #ifndef MSD_GEN16_MIN_ROWS
@@ -1486,7 +1488,21 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   // A few key tiles per query tile (cross attention over a short text): the launch is mostly reading Q and writing O,
   // and two 4-wave workgroups per CU overlap one's memory phases with the other's tiles better than one 8-wave
   // workgroup does (75600 queries x 40 heads: 0.42 vs 0.53 ms at 77 keys, 0.62 vs 0.70 at 226, equal at 512).
-  if (Skv <= kShortKv) {
+  // Grids of 256-row workgroups that fill the 256 CUs badly - at most half of them busy, or a second round for at
+  // most half of them - run as 128-row workgroups of four waves, two to a CU, on the same 4-wave kernel: it reaches
+  // 86 % of the 8-wave kernel's rate on a full chip, and B x N = 16: S 1024 / 1536 / 2048 31 -> 25, 43 -> 35,
+  // 56 -> 46 us, S 4608 (288 workgroups of 256 rows) 218 -> 206 us; 24 heads at S 3072: 152 -> 139 us.  (In between
+  // - 129 .. 256 workgroups - and from 385 on the 8-wave kernel is faster.  At head_dim 64 the alternative is
+  // fa_hd_kernel at 81 % of the rate: no gain, the rule is head_dim 128's alone.)
+  // MINDIESD_DENSE_TILE_ROWS = 256 or 128 in the environment overrides the choice of this paragraph (the tests reach
+  // both kernels at every size that way).
+  const long long tiles256 = (long long)B * N * ((Sq + 255) / 256);
+  bool half_tiles = 2 * tiles256 <= kCus || (tiles256 > kCus && 2 * tiles256 <= 3 * kCus);
+  if (const char* rows = getenv("MINDIESD_DENSE_TILE_ROWS")) {
+    if (atoi(rows) == 256) half_tiles = false;
+    if (atoi(rows) == 128) half_tiles = true;
+  }
+  if (Skv <= kShortKv || half_tiles) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
   }

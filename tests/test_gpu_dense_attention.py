@@ -12,6 +12,16 @@ MAX_ABS = 2e-2
 MIN_COS = 0.9999
 
 
+@pytest.fixture(autouse=True, params=["auto", "256", "128"])
+def dense_tile_rows(request, monkeypatch):
+    """Every test of this file under the library's own choice between its 256-row (8 waves) and 128-row (4 waves)
+    kernels at head_dim 128 - made from how the grid fills the chip - and with either forced."""
+    if request.param == "auto":
+        monkeypatch.delenv("MINDIESD_DENSE_TILE_ROWS", raising=False)
+    else:
+        monkeypatch.setenv("MINDIESD_DENSE_TILE_ROWS", request.param)
+
+
 def _qkv(shape, seed, dtype=torch.bfloat16, mul=1.0, kv_shape=None):
     g = torch.Generator().manual_seed(seed)
     q = (torch.randn(shape, generator=g) * mul).to(dtype)

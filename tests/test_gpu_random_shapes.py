@@ -28,9 +28,13 @@ def _heads(r):
 
 
 @pytest.mark.parametrize("seed", range(48))
-def test_dense_random_shape(cuda, seed):
+def test_dense_random_shape(cuda, seed, monkeypatch):
     import mindiesd
     r = random.Random(seed)
+    # (head_dim 128: the library picks 256- or 128-row workgroups from how the grid fills the chip; odd seeds force
+    # the 256-row kernel, which these small grids would not reach otherwise)
+    if seed % 2:
+        monkeypatch.setenv("MINDIESD_DENSE_TILE_ROWS", "256")
     d = r.choice([128, 128, 64, 32, 96, 256])
     sq = r.choice(SQ)
     skv = sq if r.random() < 0.5 else r.choice(SKV)
@@ -96,7 +100,7 @@ def test_masked_or_causal_random_shape(cuda, seed):
 
 
 @pytest.mark.parametrize("seed", range(40))
-def test_long_random_shape(cuda, seed):
+def test_long_random_shape(cuda, seed, monkeypatch):
     """Long sequences, where dense, causal, key-mask and packed calls run on the 16x16x32 kernels at every
     head_dim (padded where it is not 64, 128 or 256): random lengths off the tile sizes, head dims of every kernel,
     grouped-query heads, both dtypes."""
@@ -104,6 +108,8 @@ def test_long_random_shape(cuda, seed):
     from mindiesd.layers.flash_attn.hip_flash_attn import flash_attention
     from oracle.attention import attention_varlen
     r = random.Random(300 + seed)
+    if seed % 2:
+        monkeypatch.setenv("MINDIESD_DENSE_TILE_ROWS", "256")   # (see test_dense_random_shape)
     d = r.choice([40, 64, 72, 96, 128, 128, 160, 256])
     mode = r.choice(["dense", "causal", "keymask", "varlen", "varlen_causal"])
     sq, skv = r.randrange(1024, 2400), r.randrange(385, 2600)
