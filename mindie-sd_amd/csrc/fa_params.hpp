@@ -179,13 +179,13 @@ inline long long fa16_grid(const FaParams& p, int rows) {
 int launch_fa_hd(const FaParams& p, int dtype, int D, hipStream_t stream);
 
 // Attention at head_dim 64 exactly (flash_attn_d64.hip); `gen` as the GEN of fa_fwd16_kernel: 0 dense, 1 p.seq_meta
-// and / or causal, 2 the same with p.packed_tiles (256-row tiles), 3 a mask row shared by all queries.  `supported`
-// is false when a K or V (batch, head) slice does not fit the kernel's 32-bit buffer offsets (the general kernel
-// takes those).
+// and / or causal, 2 the same with p.packed_tiles (256-row tiles), 3 a mask row shared by all queries.  `rows`: query
+// rows per workgroup, 256 (8 waves) or - gen 0 only - 128 (4 waves, two workgroups per CU).  `supported` is false
+// when a K or V (batch, head) slice does not fit the kernel's 32-bit buffer offsets (the general kernel takes those).
 bool fa16_d64_supported(const FaParams& p);
-int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen = 0);
+int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen = 0, int rows = 256);
 // head dims below 64 (multiples of 8), computed as 64
-int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen = 0);
+int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen = 0, int rows = 256);
 
 // Attention at head dims above 128 up to 256 (flash_attn_d256.hip; multiples of 8, computed as 256); `gen` as for
 // launch_fa16_d64 (its packed tiles are 128 rows); `supported` as above.

@@ -125,14 +125,16 @@ constexpr int kD64Ahead = 3;                          // K operand groups reques
 // DPAD: head dims below 64 (p.head_dim, a multiple of 8) computed as 64: the query operand is zero from
 // the real head_dim on, the lanes that would stage the 16-byte chunks of K and V past it request an offset beyond
 // the buffers' range (the DMA writes zeros for them without touching memory), output columns past it are not stored.
-template <int DT, int GEN = 0, bool DPAD = false>
-__global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const FaParams p) {
+// NW: waves per workgroup, 32 query rows each - 8 (one workgroup per CU), or 4 (two per CU: for grids that fill the
+// chip badly as 256-row workgroups).
+template <int DT, int GEN = 0, bool DPAD = false, int NW = kD64Waves>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void fa_fwd16_d64_kernel(const FaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using namespace d64;
   using E = Elem<DT>;
   using T = typename E::type;
   using X8 = typename E::x8;
-  constexpr int NWAVES = kD64Waves, BN = kD64BN, kBM = NWAVES * 32, kRowBytes = kD64RowBytes;
+  constexpr int NWAVES = NW, BN = kD64BN, kBM = NWAVES * 32, kRowBytes = kD64RowBytes;
   constexpr int kTileBytes = kD64TileBytes, kORowBytes = kRowBytes + 8;
   static_assert(NWAVES * 32 * kORowBytes <= kD64Lds, "the output staging reuses the tile stages");
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -489,14 +491,14 @@ __global__ __launch_bounds__(kD64Waves * 64, 1) void fa_fwd16_d64_kernel(const F
 }
 
 
-template <int DT, int GEN, bool DPAD = false>
+template <int DT, int GEN, bool DPAD = false, int NW = kD64Waves>
 static int launch_d64(const FaParams& p, hipStream_t stream) {
-  auto kern = fa_fwd16_d64_kernel<DT, GEN, DPAD>;
+  auto kern = fa_fwd16_d64_kernel<DT, GEN, DPAD, NW>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kD64Lds) != hipSuccess)
     return MSD_ERR_LAUNCH;
-  const long long grid = fa16_grid<GEN, false>(p, kD64Waves * 32);
+  const long long grid = fa16_grid<GEN, false>(p, NW * 32);
   if (grid > 0x7ffffff0ll) return MSD_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kD64Waves * 64), kD64Lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), kD64Lds, stream, p);
   return hipGetLastError() == hipSuccess ? MSD_OK : MSD_ERR_LAUNCH;
 }
 
@@ -506,11 +508,14 @@ bool fa16_d64_supported(const FaParams& p) {
   return (long long)p.Skv * p.k_ss * 2 < 0x7fffff00ll && (long long)p.Skv * p.v_ss * 2 < 0x7fffff00ll;
 }
 
-int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen) {
+int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stream, int gen, int rows) {
   if (!fa16_d64_supported(p) || D <= 0 || D >= 64 || (D & 7) || gen < 0 || gen > 3) return MSD_ERR_UNSUPPORTED;
+  if (rows != 256 && !(rows == 128 && gen == 0)) return MSD_ERR_UNSUPPORTED;
   FaParams pp = p;
   pp.head_dim = D;
   const bool bf = dtype == MSD_DTYPE_BF16;
+  if (rows == 128)
+    return bf ? launch_d64<MSD_DTYPE_BF16, 0, true, 4>(pp, stream) : launch_d64<MSD_DTYPE_F16, 0, true, 4>(pp, stream);
   switch (gen) {
     case 1: return bf ? launch_d64<MSD_DTYPE_BF16, 1, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 1, true>(pp, stream);
     case 2: return bf ? launch_d64<MSD_DTYPE_BF16, 2, true>(pp, stream) : launch_d64<MSD_DTYPE_F16, 2, true>(pp, stream);
@@ -519,9 +524,12 @@ int launch_fa16_d64_padded(const FaParams& p, int dtype, int D, hipStream_t stre
   }
 }
 
-int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen) {
+int launch_fa16_d64(const FaParams& p, int dtype, hipStream_t stream, int gen, int rows) {
   if (!fa16_d64_supported(p) || gen < 0 || gen > 3) return MSD_ERR_UNSUPPORTED;
+  if (rows != 256 && !(rows == 128 && gen == 0)) return MSD_ERR_UNSUPPORTED;
   const bool bf = dtype == MSD_DTYPE_BF16;
+  if (rows == 128)
+    return bf ? launch_d64<MSD_DTYPE_BF16, 0, false, 4>(p, stream) : launch_d64<MSD_DTYPE_F16, 0, false, 4>(p, stream);
   switch (gen) {
     case 1: return bf ? launch_d64<MSD_DTYPE_BF16, 1>(p, stream) : launch_d64<MSD_DTYPE_F16, 1>(p, stream);
     case 2: return bf ? launch_d64<MSD_DTYPE_BF16, 2>(p, stream) : launch_d64<MSD_DTYPE_F16, 2>(p, stream);

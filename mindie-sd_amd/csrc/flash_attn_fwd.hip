@@ -1470,7 +1470,17 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   const int rc = check_common(q, k, v, out, dtype, B, N, Nkv, Sq, Skv, D, st, scale, true);
   if (rc != MSD_OK) return rc;
   FaParams p = make_params(q, k, v, out, lse, B, N, Nkv, Sq, Skv, st, scale);
-  if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream);
+  // Grids of 256-row workgroups that fill the 256 CUs badly - at most half of them busy, or a second round for at
+  // most half of them - run as 128-row workgroups of four waves, two to a CU (head dims 128 and up to 64).
+  // MINDIESD_DENSE_TILE_ROWS = 256 or 128 in the environment overrides the choice (the tests reach both kinds of
+  // kernel at every size that way).
+  const long long tiles256 = (long long)B * N * ((Sq + 255) / 256);
+  bool half_tiles = 2 * tiles256 <= kCus || (tiles256 > kCus && 2 * tiles256 <= 3 * kCus);
+  if (const char* rows = getenv("MINDIESD_DENSE_TILE_ROWS")) {
+    if (atoi(rows) == 256) half_tiles = false;
+    if (atoi(rows) == 128) half_tiles = true;
+  }
+  if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream, 0, half_tiles ? 128 : 256);
   // Head dims between 64 and 128 run as head_dim 128 on the 16x16x32 kernel (the part of the matrix work spent on
   // the padding costs less than the general kernel's staging through registers: 72 -> 580 vs 730 TFLOP/s of real
   // work, 112 -> 800 vs 1130), when the 256-byte rows the DMA fetches stay inside the kernel's 32-bit offsets.
@@ -1483,25 +1493,15 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   // (the rule for short key sequences below is head_dim 128's alone: at the other widths the alternative is the
   // general kernel, which these beat at 77 keys already)
   if (D > 128 && fa16_d256_supported(p)) return launch_fa16_d256(p, dtype, D, stream);
-  if (D < 64 && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream);
+  if (D < 64 && fa16_d64_supported(p)) return launch_fa16_d64_padded(p, dtype, D, stream, 0, half_tiles ? 128 : 256);
   if (D != 128) return launch_fa_hd(p, dtype, D, stream);
   // A few key tiles per query tile (cross attention over a short text): the launch is mostly reading Q and writing O,
   // and two 4-wave workgroups per CU overlap one's memory phases with the other's tiles better than one 8-wave
   // workgroup does (75600 queries x 40 heads: 0.42 vs 0.53 ms at 77 keys, 0.62 vs 0.70 at 226, equal at 512).
-  // Grids of 256-row workgroups that fill the 256 CUs badly - at most half of them busy, or a second round for at
-  // most half of them - run as 128-row workgroups of four waves, two to a CU, on the same 4-wave kernel: it reaches
-  // 86 % of the 8-wave kernel's rate on a full chip, and B x N = 16: S 1024 / 1536 / 2048 31 -> 25, 43 -> 35,
-  // 56 -> 46 us, S 4608 (288 workgroups of 256 rows) 218 -> 206 us; 24 heads at S 3072: 152 -> 139 us.  (In between
-  // - 129 .. 256 workgroups - and from 385 on the 8-wave kernel is faster.  At head_dim 64 the alternative is
-  // fa_hd_kernel at 81 % of the rate: no gain, the rule is head_dim 128's alone.)
-  // MINDIESD_DENSE_TILE_ROWS = 256 or 128 in the environment overrides the choice of this paragraph (the tests reach
-  // both kernels at every size that way).
-  const long long tiles256 = (long long)B * N * ((Sq + 255) / 256);
-  bool half_tiles = 2 * tiles256 <= kCus || (tiles256 > kCus && 2 * tiles256 <= 3 * kCus);
-  if (const char* rows = getenv("MINDIESD_DENSE_TILE_ROWS")) {
-    if (atoi(rows) == 256) half_tiles = false;
-    if (atoi(rows) == 128) half_tiles = true;
-  }
+  // The same 4-wave kernel takes the grids that fill the chip badly (half_tiles above): it reaches 86 % of the 8-wave
+  // kernel's rate on a full chip, and B x N = 16: S 1024 / 1536 / 2048 31 -> 25, 43 -> 35, 56 -> 46 us, S 4608 (288
+  // workgroups of 256 rows) 218 -> 206 us; 24 heads at S 3072: 152 -> 139 us.  (In between - 129 .. 256 workgroups -
+  // and from 385 on the 8-wave kernel is faster.)
   if (Skv <= kShortKv || half_tiles) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa<MSD_DTYPE_BF16, 4, 32, 64, false, 1, 1>(p, stream);
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 1>(p, stream);
