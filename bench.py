@@ -194,6 +194,35 @@ def extra_head_dims(device, steps, warmup):
     return res
 
 
+def extra_mid_size_grids(device, steps, warmup):
+    """Dense calls whose grid fills the 256 CUs badly as 256-row workgroups (few heads, a few thousand tokens): the
+    entry point runs them as 128-row workgroups; both choices timed (MINDIESD_DENSE_TILE_ROWS forces either)."""
+    import os
+    import torch
+    import mindiesd
+    res = {"workload": "dense bf16 B1: N16 S2048 D128, N24 S3072 D128, N16 S4608 D128, N24 S4096 D64 "
+                       "(128, 288, 288 and 384 workgroups of 256 rows)"}
+    keep = os.environ.get("MINDIESD_DENSE_TILE_ROWS")
+    try:
+        for n, s, d in ((16, 2048, 128), (24, 3072, 128), (16, 4608, 128), (24, 4096, 64)):
+            g = torch.Generator(device=device).manual_seed(13)
+            q, k, v = ((torch.randn((1, n, s, d), device=device, generator=g) * 0.5).to(torch.bfloat16) for _ in range(3))
+            for rows in ("auto", "256"):
+                os.environ.pop("MINDIESD_DENSE_TILE_ROWS", None)
+                if rows != "auto":
+                    os.environ["MINDIESD_DENSE_TILE_ROWS"] = rows
+                ms, _ = time_steps(lambda: mindiesd.attention_forward(q, k, v, head_first=True), max(steps, 10), max(warmup, 3))
+                m = median(ms)
+                key = f"n{n}_s{s}_d{d}" + ("" if rows == "auto" else "_256_rows_forced")
+                res[key + "_us"] = 1e3 * m
+                res[key + "_tflops"] = 4.0 * n * s * s * d / m / 1e9
+    finally:
+        os.environ.pop("MINDIESD_DENSE_TILE_ROWS", None)
+        if keep is not None:
+            os.environ["MINDIESD_DENSE_TILE_ROWS"] = keep
+    return res
+
+
 def extra_cross_attention(device, steps, warmup):
     """Dense attention of the 720p video tokens over a short text (few key tiles per query tile: the launch is
     mostly reading Q and writing O)."""
@@ -506,6 +535,7 @@ def main():
         extras = {}
         for name, fn in (("dense_wan1p3b", lambda: extra_dense_1p3b(device, args.steps, args.warmup)),
                          ("head_dims", lambda: extra_head_dims(device, args.steps, args.warmup)),
+                         ("mid_size_grids", lambda: extra_mid_size_grids(device, args.steps, args.warmup)),
                          ("cross_attention", lambda: extra_cross_attention(device, args.steps, args.warmup)),
                          ("causal_varlen", lambda: extra_causal_varlen(device, args.steps, args.warmup)),
                          ("sparse_rf_v3", lambda: extra_sparse(device, args.steps, args.warmup, kernel_ms)),
