@@ -82,7 +82,29 @@ def check(rc, what):
 
 
 def stream_ptr(device=None):
+    """The current HIP stream of ``device`` as an integer handle."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None and device is not None and device.index is not None:
+        return raw(device.index)                      # (no Stream object: a microsecond less per call)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _Here:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_HERE = _Here()
+
+
+def on_device(device):
+    """Context that makes ``device`` the current one for the launch; nothing to do when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _HERE
+    return torch.cuda.device(device)
 
 
 DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}

@@ -45,7 +45,7 @@ def sparse_block_estimate(query, key, input_layout="BNSD", stride=8, sparse_size
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
     mask = torch.empty((b, n, nb, pitch), dtype=torch.int8, device=q.device)
     count = torch.empty((b, n, nb), dtype=torch.int32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         stream = _native.stream_ptr(q.device)
         rc = lib.mindiesd_sbe_scores(q.data_ptr(), k.data_ptr(), scores.data_ptr(), _native.DTYPE_CODE[q.dtype], b, n,
                                      nkv, s, HEAD_DIM, *_strides_bns(q, input_layout), *_strides_bns(k, input_layout),
@@ -87,7 +87,7 @@ def ada_block_sparse_attention(query, key, value, sparse_mask, sparse_count_tabl
         return block_sparse_attention_mask(q, k, v, sparse_mask[..., :nb], scale_value, input_layout)
     idx, cnt = mask_to_lists(sparse_mask)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         rc = _native.lib().mindiesd_ada_block_sparse_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _native.DTYPE_CODE[q.dtype], b, n, nkv, s,
             q.shape[-1], *_strides_bns(q, input_layout), *_strides_bns(k, input_layout), *_strides_bns(v, input_layout),

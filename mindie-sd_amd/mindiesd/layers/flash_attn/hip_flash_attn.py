@@ -18,11 +18,10 @@ MAX_HEAD_DIM = 256    # dense attention takes every multiple of 8 up to this
 
 def _strides_bns(t, layout):
     """(batch, head, token) element strides of a 4-D tensor in ``layout`` with a contiguous last dim."""
-    if t.stride(-1) != 1:
+    s0, s1, s2, s3 = t.stride()
+    if s3 != 1:
         raise ParametersInvalid("The last dimension of query/key/value must be contiguous.")
-    if layout == "BNSD":
-        return t.stride(0), t.stride(1), t.stride(2)
-    return t.stride(0), t.stride(2), t.stride(1)
+    return (s0, s1, s2) if layout == "BNSD" else (s0, s2, s1)
 
 
 def _check_qkv(query, key, value):
@@ -39,8 +38,13 @@ def _check_qkv(query, key, value):
 
 
 def _aligned(t):
-    return t if (t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1])
-                 and t.data_ptr() % 16 == 0) else t.contiguous()
+    st = t.stride()
+    if st[-1] != 1 or t.data_ptr() % 16:
+        return t.contiguous()
+    for s in st[:-1]:
+        if s % 8:
+            return t.contiguous()
+    return t
 
 
 def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, attn_mask=None, causal=False):
@@ -65,7 +69,7 @@ def flash_attention(query, key, value, scale, layout="BNSD", return_lse=False, a
     lse = torch.empty((b, n, sq), dtype=torch.float32, device=query.device) if return_lse else None
     strides = (*_strides_bns(query, layout), *_strides_bns(key, layout), *_strides_bns(value, layout),
                *_strides_bns(out, layout))
-    with torch.cuda.device(query.device):
+    with _native.on_device(query.device):
         if attn_mask is None and not causal:
             rc = _native.lib().mindiesd_flash_attention_fwd(
                 query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(),
@@ -115,7 +119,7 @@ def _varlen_meta(cu_q, cu_k, total_q, total_k, device, max_q=None, max_k=None):
         bound_q = total_q if max_q is None else max(min(int(max_q), total_q), 1)
         bound_k = total_k if max_k is None else max(min(int(max_k), total_k), 0)
         meta = torch.empty((cq.shape[0] - 1, 4), dtype=torch.int32, device=device)
-        with torch.cuda.device(device):
+        with _native.on_device(device):
             rc = _native.lib().mindiesd_varlen_meta(cq.data_ptr(), ck.data_ptr(), cq.shape[0] - 1, total_q, total_k,
                                                     bound_q, bound_k, meta.data_ptr(), _native.stream_ptr(device))
         _native.check(rc, "mindiesd_varlen_meta")
@@ -163,7 +167,7 @@ def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=Fa
     tn = lambda t: (0, t.stride(1), t.stride(0))  # (batch, head, token) strides of a [T, N, D] tensor
     if unchecked and max_seqlen_q is None and max_seqlen_k is None:
         # lengths known to the device only: the grid comes from the token totals, the workgroups find their sequence
-        with torch.cuda.device(q.device):
+        with _native.on_device(q.device):
             rc = _native.lib().mindiesd_flash_attention_packed_fwd(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _native.DTYPE_CODE[q.dtype],
                 nseq, q.shape[1], k.shape[1], q.shape[0], k.shape[0], q.shape[2],
@@ -171,7 +175,7 @@ def flash_attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, scale, causal=Fa
                 _native.stream_ptr(q.device))
         _native.check(rc, "mindiesd_flash_attention_packed_fwd")
         return out
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         rc = _native.lib().mindiesd_flash_attention_general_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None, _native.DTYPE_CODE[q.dtype],
             nseq, q.shape[1], k.shape[1], max_q, max_k, q.shape[2],

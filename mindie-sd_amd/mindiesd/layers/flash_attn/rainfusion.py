@@ -63,7 +63,7 @@ def _run_rearrange(srcs, dsts, pool, layout, grid, txt_len, inverse):
         pst = b * pool.stride(0)
     else:
         pst = psb = psn = psblk = 0
-    with torch.cuda.device(x.device):
+    with _native.on_device(x.device):
         rc = _native.lib().mindiesd_rf_rearrange_pool(
             ptr(srcs, 0), ptr(srcs, 1), ptr(srcs, 2), ptr(dsts, 0), ptr(dsts, 1), ptr(dsts, 2),
             pool.data_ptr() if pool is not None else None, _native.DTYPE_CODE[x.dtype], b, n, s, x.shape[-1],
@@ -205,7 +205,7 @@ def get_mask_index(mask):
     m8 = mask.to(torch.int8).contiguous()
     idx = torch.empty((b, n, qb, kb), dtype=torch.int32, device=mask.device)
     cnt = torch.empty((b, n, qb), dtype=torch.int32, device=mask.device)
-    with torch.cuda.device(mask.device):
+    with _native.on_device(mask.device):
         rc = _native.lib().mindiesd_mask_to_index(m8.data_ptr(), b * n, qb, kb, idx.data_ptr(), cnt.data_ptr(), kb,
                                                   _native.stream_ptr(mask.device))
     _native.check(rc, "mindiesd_mask_to_index")
@@ -241,7 +241,7 @@ def _block_mask(qkv_pool, txt_len, sparsity, scale, pool_size, latent_shape_q, i
     sel_num = torch.empty((nb, n), dtype=torch.int64, device=dev) if want_ref_lists else None
     qp, kp = pool[:b], pool[b:2 * b]
     p = lambda t: t.data_ptr() if t is not None else None
-    with torch.cuda.device(dev):
+    with _native.on_device(dev):
         rc = _native.lib().mindiesd_rf_block_mask(
             qp.data_ptr(), kp.data_ptr(), _native.DTYPE_CODE[pool.dtype], b, n, nb, pool.shape[-1],
             *_pool_strides(qp, input_layout), float(scale), keep_len, txt_blocks, ff_blocks, int(bool(keep_diagonal)),
@@ -276,7 +276,7 @@ _token_order_lock = threading.Lock()
 def _build_token_order(t, h, w, txt_len, dev):
     s = t * h * w + txt_len
     tok = torch.empty((s,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _native.on_device(dev):
         rc = _native.lib().mindiesd_rf_token_order(tok.data_ptr(), s, t, h, w, txt_len, _native.stream_ptr(dev))
     _native.check(rc, "mindiesd_rf_token_order")
     return tok
@@ -347,7 +347,7 @@ def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, lay
                 or order.device != q.device):
             raise ParametersInvalid(f"order must be a contiguous int32 [{sq}] tensor on the inputs' device "
                                     "(self-attention only).")
-        with torch.cuda.device(q.device):
+        with _native.on_device(q.device):
             rc = _native.lib().mindiesd_block_sparse_attention_gather_fwd(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
                 _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, q.shape[-1],
@@ -356,7 +356,7 @@ def block_sparse_attention_lists(query, key, value, blk_idx, blk_cnt, scale, lay
                 _native.stream_ptr(q.device))
         _native.check(rc, "mindiesd_block_sparse_attention_gather_fwd")
         return (out, lse) if return_lse else out
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         rc = _native.lib().mindiesd_block_sparse_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
             _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1],
@@ -396,7 +396,7 @@ def block_sparse_attention_mask(query, key, value, block_sparse_mask, scale, lay
     lse = torch.empty((b, n, sq), dtype=torch.float32, device=q.device) if return_lse else None
     ws_bytes = lib.mindiesd_block_sparse_attention_paired_workspace_size(b, n, sq, skv)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         rc = lib.mindiesd_block_sparse_attention_paired_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
             _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1],
@@ -459,7 +459,7 @@ def block_sparse_attention_varlen(query, key, value, block_sparse_mask, scale, s
     idx, cnt = mask_to_lists(block_sparse_mask[:, :, :qb, :kb])
     meta = torch.tensor([[starts_q[i], lq[i], starts_k[i], lk[i]] for i in range(b)], dtype=torch.int32).to(q.device)
     o_str = (0, out.stride(1), out.stride(0)) if layout == "TND" else _strides_bns(out, layout)
-    with torch.cuda.device(q.device):
+    with _native.on_device(q.device):
         rc = _native.lib().mindiesd_block_sparse_attention_general_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr() if return_lse else None,
             _native.DTYPE_CODE[q.dtype], b, n, nkv, sq, skv, q.shape[-1], *q_str, *k_str, *v_str, *o_str, float(scale),
@@ -477,7 +477,7 @@ def mask_to_lists(block_sparse_mask):
     b, n, qb, kb = m8.shape
     idx = torch.empty((b, n, qb, kb), dtype=torch.int32, device=m8.device)
     cnt = torch.empty((b, n, qb), dtype=torch.int32, device=m8.device)
-    with torch.cuda.device(m8.device):
+    with _native.on_device(m8.device):
         rc = _native.lib().mindiesd_mask_to_index(m8.data_ptr(), b * n, qb, kb, idx.data_ptr(), cnt.data_ptr(), kb,
                                                   _native.stream_ptr(m8.device))
     _native.check(rc, "mindiesd_mask_to_index")

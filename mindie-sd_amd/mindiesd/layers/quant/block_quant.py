@@ -21,7 +21,7 @@ def _block_quant(x, block_size, layout, prescale=1.0, pow2=False):
     b, n, s = (x.shape[0], x.shape[1], x.shape[2]) if layout == "BNSD" else (x.shape[0], x.shape[2], x.shape[1])
     q = torch.empty((b, n, s, HEAD_DIM), dtype=torch.uint8, device=x.device)
     scale = torch.empty((b, n, (s + block_size - 1) // block_size), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _native.on_device(x.device):
         rc = _native.lib().mindiesd_fa_block_quant(x.data_ptr(), q.data_ptr(), scale.data_ptr(),
                                                    _native.DTYPE_CODE[x.dtype], b, n, s, HEAD_DIM,
                                                    *_strides_bns(x, layout), block_size, float(prescale),
@@ -45,7 +45,7 @@ def _rot_block_quant(x, rot, layout, prescale=1.0, pow2=False):
     b, n, s = (x.shape[0], x.shape[1], x.shape[2]) if layout == "BNSD" else (x.shape[0], x.shape[2], x.shape[1])
     q = torch.empty((b, n, s, HEAD_DIM), dtype=torch.uint8, device=x.device)
     scale = torch.empty((b, n, (s + 127) // 128), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _native.on_device(x.device):
         rc = _native.lib().mindiesd_fa_rot_block_quant(x.data_ptr(), rot_t.data_ptr(), q.data_ptr(), scale.data_ptr(),
                                                        _native.DTYPE_CODE[x.dtype], b, n, s, HEAD_DIM,
                                                        *_strides_bns(x, layout), float(prescale), int(bool(pow2)),

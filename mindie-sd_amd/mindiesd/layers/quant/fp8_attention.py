@@ -25,7 +25,7 @@ def quantize_v_per_channel(value, layout="BNSD"):
     vscale = torch.empty((b, n, HEAD_DIM), dtype=torch.float32, device=v.device)
     lib = _native.lib()
     ws = torch.empty(lib.mindiesd_fp8_v_quant_workspace_size(b, n), dtype=torch.uint8, device=v.device)
-    with torch.cuda.device(v.device):
+    with _native.on_device(v.device):
         rc = lib.mindiesd_fp8_v_quant(v.data_ptr(), v8t.data_ptr(), vscale.data_ptr(), _native.DTYPE_CODE[v.dtype],
                                       b, n, s, HEAD_DIM, *_strides_bns(v, layout), ws.data_ptr(), ws.numel(),
                                       _native.stream_ptr(v.device))
@@ -57,7 +57,7 @@ def fp8_attention_quantized(q8, q_scale, k8, k_scale, v8t, v_scale, scale, out_d
     skv = k8.shape[2]
     shape = (b, n, sq, d) if layout == "BNSD" else (b, sq, n, d)
     out = torch.empty(shape, dtype=out_dtype, device=q8.device)
-    with torch.cuda.device(q8.device):
+    with _native.on_device(q8.device):
         rc = _native.lib().mindiesd_fp8_attention_fwd(
             q8.data_ptr(), k8.data_ptr(), v8t.data_ptr(), q_scale.data_ptr(), k_scale.data_ptr(), v_scale.data_ptr(),
             out.data_ptr(), _native.DTYPE_CODE[out_dtype], b, n, sq, skv, d, *_strides_bns(out, layout),

@@ -22,7 +22,7 @@ def mx_quantize(x):
         x = x.contiguous()
     q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
     e = torch.empty((m, k // 32), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _native.on_device(x.device):
         rc = _native.lib().mindiesd_mx_quant(x.data_ptr(), q.data_ptr(), e.data_ptr(), _native.DTYPE_CODE[x.dtype], m, k,
                                              x.stride(0), _native.stream_ptr(x.device))
     _native.check(rc, "mindiesd_mx_quant")
@@ -58,7 +58,7 @@ def mxfp8_matmul(x_q, x_scale, w_q, w_scale, bias=None, out_dtype=torch.bfloat16
         if bias.numel() != nw:
             raise ParametersInvalid("bias must have one entry per weight row.")
     out = torch.empty((m, nw // 2 if swiglu else nw), dtype=out_dtype, device=xq.device)
-    with torch.cuda.device(xq.device):
+    with _native.on_device(xq.device):
         rc = _native.lib().mindiesd_mxfp8_gemm(xq.data_ptr(), xs.data_ptr(), wq.data_ptr(), ws.data_ptr(),
                                                bias.data_ptr() if bias is not None else None, out.data_ptr(),
                                                _native.DTYPE_CODE[out_dtype], m, k, nw, int(bool(swiglu)),
