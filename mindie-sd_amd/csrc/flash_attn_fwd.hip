@@ -1461,6 +1461,17 @@ int mindiesd_block_sparse_attention_paired_fwd(const void* q, const void* k, con
                      : launch_fa<MSD_DTYPE_F16, 4, 32, 64, true, 1, 0, false, true>(p, stream);
 }
 
+// True when B x N x ceil(Sq / 256) workgroups of 256 rows would fill the chip badly (see mindiesd_flash_attention_fwd).
+static bool prefers_half_tiles(int B, int N, int Sq) {
+  const long long tiles256 = (long long)B * N * ((Sq + 255) / 256);
+  bool half_tiles = 2 * tiles256 <= kCus || (tiles256 > kCus && 2 * tiles256 <= 3 * kCus);
+  if (const char* rows = getenv("MINDIESD_DENSE_TILE_ROWS")) {
+    if (atoi(rows) == 256) half_tiles = false;
+    if (atoi(rows) == 128) half_tiles = true;
+  }
+  return half_tiles;
+}
+
 int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
                                  int B, int N, int Nkv, int Sq, int Skv, int D, long long q_sb, long long q_sn,
                                  long long q_ss, long long k_sb, long long k_sn, long long k_ss, long long v_sb,
@@ -1474,12 +1485,7 @@ int mindiesd_flash_attention_fwd(const void* q, const void* k, const void* v, vo
   // most half of them - run as 128-row workgroups of four waves, two to a CU (head dims 128 and up to 64).
   // MINDIESD_DENSE_TILE_ROWS = 256 or 128 in the environment overrides the choice (the tests reach both kinds of
   // kernel at every size that way).
-  const long long tiles256 = (long long)B * N * ((Sq + 255) / 256);
-  bool half_tiles = 2 * tiles256 <= kCus || (tiles256 > kCus && 2 * tiles256 <= 3 * kCus);
-  if (const char* rows = getenv("MINDIESD_DENSE_TILE_ROWS")) {
-    if (atoi(rows) == 256) half_tiles = false;
-    if (atoi(rows) == 128) half_tiles = true;
-  }
+  const bool half_tiles = prefers_half_tiles(B, N, Sq);
   if (D == 64 && fa16_d64_supported(p)) return launch_fa16_d64(p, dtype, stream, 0, half_tiles ? 128 : 256);
   // Head dims between 64 and 128 run as head_dim 128 on the 16x16x32 kernel (the part of the matrix work spent on
   // the padding costs less than the general kernel's staging through registers: 72 -> 580 vs 730 TFLOP/s of real
@@ -1606,8 +1612,10 @@ int mindiesd_flash_attention_general_fwd(const void* q, const void* k, const voi
     return launch_fa<MSD_DTYPE_F16, 4, 32, 64, false, 1, 2>(p, stream);
   }
   // Without a mask, long sequences run on the 16x16x32 kernel's general instantiation (256-row tiles); short ones
-  // fill the chip better with the 128-row tiles of the 4-wave kernel.
-  if (long_rows) {
+  // fill the chip better with the 128-row tiles of the 4-wave kernel, and so do causal calls whose grid of 256-row
+  // workgroups would fill it badly (the rule of mindiesd_flash_attention_fwd; B x N 16: S 1024 / 2048 32 -> 25,
+  // 54 -> 42 us, 48 heads at S 2048 82 -> 75 us).
+  if (long_rows && !(causal && !seq_meta && prefers_half_tiles(B, N, Sq))) {
     if (dtype == MSD_DTYPE_BF16) return launch_fa16<MSD_DTYPE_BF16, 8, false, false, 1>(p, stream);
     return launch_fa16<MSD_DTYPE_F16, 8, false, false, 1>(p, stream);
   }

@@ -9,6 +9,17 @@ from oracle.attention import attention_math, attention_varlen, causal_keep_mask,
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "256"])
+def dense_tile_rows(request, monkeypatch):
+    """Causal calls at head_dim 128 choose between the 256-row general kernel and the 128-row one from how the grid
+    fills the chip; every test of this file runs under that choice and with the 256-row kernels forced (these small
+    grids would not reach them otherwise)."""
+    if request.param == "auto":
+        monkeypatch.delenv("MINDIESD_DENSE_TILE_ROWS", raising=False)
+    else:
+        monkeypatch.setenv("MINDIESD_DENSE_TILE_ROWS", request.param)
+
+
 def _rand(shape, seed, dtype=torch.bfloat16, mul=1.0):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(shape, generator=g) * mul).to(dtype)
